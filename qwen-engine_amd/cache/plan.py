@@ -10,10 +10,13 @@ from .manager import GroupSpec
 
 @dataclass(frozen=True)
 class KVNeed:
-    """Keys and values of every position (window None) or of the last ``window``."""
+    """Keys and values of every position (window None) or of the last ``window``.  ``planes``: 2 for a
+    key and a value tile per head and page; 1 for a part that keeps one row per token (a latent from
+    which it forms both)."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    planes: int = 2
 
 
 @dataclass(frozen=True)
@@ -37,7 +40,7 @@ class CachePlan:
     user_state: List[Optional[StateNeed]]    # per user: fixed-size state
 
     def bytes_per_token(self, itemsize: int) -> int:
-        return sum(2 * kv.num_kv_heads * kv.head_dim * itemsize for kv in self.user_kv if kv is not None)
+        return sum(kv.planes * kv.num_kv_heads * kv.head_dim * itemsize for kv in self.user_kv if kv is not None)
 
 
 Need = Tuple[Optional[KVNeed], Optional[StateNeed]]
@@ -68,7 +71,7 @@ def plan_cache(entry_needs: Sequence[tuple]) -> CachePlan:
                 src = entry_users[cache_from][j]
                 src_kv = user_kv[src]
                 if kv is not None and src_kv is not None and \
-                        (kv.num_kv_heads, kv.head_dim) != (src_kv.num_kv_heads, src_kv.head_dim):
+                        (kv.num_kv_heads, kv.head_dim, kv.planes) != (src_kv.num_kv_heads, src_kv.head_dim, src_kv.planes):
                     raise ValueError(f"schedule entry {i} cannot read the cache of entry {cache_from}: "
                                      f"their key/value shapes differ")
                 if kv is not None and src_kv is not None and src_kv.window is not None and \

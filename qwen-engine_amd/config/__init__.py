@@ -1,6 +1,8 @@
-from .spec import (AttentionSpec, LayerSpec, ModelSpec, RMSNormSpec, RopeSpec,
-                   ScheduleEntry, SwiGLUSpec)
+from .spec import (AttentionSpec, GroupedMoESpec, LatentAttentionSpec, LayerSpec, ModelSpec, PolyNormMLPSpec,
+                   PostNormLayerSpec, RMSNormSpec, RopePairsSpec, RopeSpec, ScalarRMSNormSpec,
+                   ScheduleEntry, ShortConvSpec, SwiGLUSpec)
 from .qwen3 import ConfigError, Qwen3Config
+from .zarorax import ZaroraxConfig
 from .registry import (config_from_dict, config_from_folder, known_architectures,
                        register_architecture, unregister_architecture)
 from .engine_config import EngineConfig

@@ -27,9 +27,9 @@ def known_architectures():
 
 
 def config_from_dict(d: Dict[str, Any]):
-    archs = d.get("architectures")
+    archs = d.get("architectures") or ([d["architecture"]] if isinstance(d.get("architecture"), str) else None)
     if not archs:
-        raise ConfigError("config.json has no 'architectures' entry; known: "
+        raise ConfigError("config.json has no 'architectures' (or 'architecture') entry; known: "
                           + ", ".join(known_architectures()))
     name = archs[0]
     if name not in _ARCHITECTURES:
@@ -47,3 +47,11 @@ def config_from_folder(folder: str):
 
 
 register_architecture(_QWEN3, Qwen3Config.from_dict)
+
+
+def _zarorax(d):
+    from .zarorax import ZaroraxConfig
+    return ZaroraxConfig.from_dict(d)
+
+
+register_architecture("Zarorax", _zarorax)

@@ -63,6 +63,94 @@ class SwiGLUSpec:
 
 
 @dataclass(frozen=True)
+class ScalarRMSNormSpec:
+    """y = g * x * rsqrt(mean(x^2) + eps) over the last dimension, g one number (a tensor of no dimensions)."""
+    eps: float
+    kind: str = "rmsnorm_scalar"
+
+
+@dataclass(frozen=True)
+class RopePairsSpec:
+    """Rotary position encoding over neighbouring pairs: the pair (2i, 2i + 1), i < rotary_dim / 2, is
+    turned by ``position * theta ** (-2 i / rotary_dim)``; features from rotary_dim on pass unchanged."""
+    theta: float
+    rotary_dim: int
+    kind: str = "rope_pairs"
+
+
+@dataclass(frozen=True)
+class ShortConvSpec:
+    """out_t = x_t + sum_j w[:, j] x_(t - taps + 1 + j): a causal convolution over time on each channel,
+    added to its input; the last ``taps - 1`` inputs of a request are state."""
+    taps: int
+    kind: str = "short_conv"
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention whose keys and values are linear maps of one cached latent per token (``kv_rank``
+    numbers, RMS-normed), with one rotated key part of ``rot_dim`` numbers shared by all heads.  A head's
+    query has ``head_dim`` unrotated and ``rot_dim`` rotated numbers, its value ``v_head_dim``.
+
+    ``q_rank`` None: queries straight from the input; else through a normed latent of that size.
+    ``output_gate``: the heads' outputs are multiplied by sigmoid of a projection of the mixer's input.
+    """
+    num_heads: int
+    head_dim: int
+    rot_dim: int
+    v_head_dim: int
+    kv_rank: int
+    scale: float
+    norm_eps: float
+    q_rank: Optional[int] = None
+    output_gate: bool = False
+    position: Optional[object] = None
+    kind: str = "latent_attention"
+
+
+@dataclass(frozen=True)
+class PolyNormMLPSpec:
+    """down(act(up x)), act(z) = a N(z) + b N(z^2) + c N(z^3) + e with N(v) = v / sqrt(mean(v^2) + eps)
+    over a token's ``intermediate_size`` values and (a, b, c, e) a tensor of the layer."""
+    intermediate_size: int
+    eps: float
+    kind: str = "polynorm_mlp"
+
+
+@dataclass(frozen=True)
+class GroupedMoESpec:
+    """A routed mixture of small gated feed-forwards.  Scores: softmax of the router's 32-bit logits over
+    all experts; the experts form ``num_groups`` equal groups of neighbours, of which the ``keep_groups``
+    with the largest best score stay; the ``top`` largest scores among those choose the experts and weigh
+    them as they are.  An expert: g = min(gate x, limit), u = clamp(up x, -limit, limit),
+    down(g * sigmoid(slope * g) * (u + 1))."""
+    num_experts: int
+    top: int
+    num_groups: int
+    keep_groups: int
+    intermediate_size: int
+    limit: float
+    slope: float = 1.702
+    kind: str = "grouped_moe"
+
+
+@dataclass(frozen=True)
+class PostNormLayerSpec:
+    """One post-norm block: x <- mixer_norm(alpha x + mixer(conv(x))); x <- ffn_norm(alpha x + ffn(x)).
+    ``conv`` (before the mixer) and ``ffn`` (with its norm) may be None.  ``names``: the checkpoint names
+    inside ``prefix`` of mixer norm, mixer, feed-forward norm, feed-forward and convolution."""
+    prefix: str
+    mixer: object
+    mixer_norm: object
+    ffn: Optional[object]
+    ffn_norm: Optional[object]
+    alpha: float
+    conv: Optional[object] = None
+    names: Tuple[str, str, str, str, str] = ("norm1", "mix", "norm2", "mlp", "canon1")
+    kind: str = "postnorm_block"
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     """One pre-norm residual block: x += mixer(norm(x)); x += ffn(norm(x)).
 

@@ -1,0 +1,253 @@
+// Mixture of experts: routing, grouping of the (token, choice) pairs by expert, and the experts'
+// two matrix products over the grouped rows.  Everything happens on the device, with grids that depend
+// on the shapes only (a block that finds no tile for itself leaves), so a step can be recorded.
+//
+//   qe_moe_route   scores = softmax(logits) over all experts (32-bit).  The experts form G equal groups
+//                  of neighbours; a group's score is its largest; only the experts of the ``keep`` best
+//                  groups can be chosen; of those the ``top`` largest are, weighted by their scores as
+//                  they are.  On ties the lower index wins.  ids [T, top], weights [T, top].
+//   qe_moe_sort    perm [T * top]: the pairs (as index t * top + j) ordered by expert; tiles
+//                  [max_tiles, 3] = (expert, first sorted row, rows <= tile_rows) and their number.
+//   qe_moe_gemm    for every tile, rows . W_e^T:
+//                    first product  (dual): x row of the pair's token against gate and up rows of
+//                      W_e [2 F, K]; g = min(g, limit), u = clamp(u, -limit, limit),
+//                      a = g sigmoid(slope g) (u + 1), stored at the sorted row
+//                    second product (weighted): a's sorted row against W_e [N, K], times the pair's
+//                      weight, to parts[j][t] (32-bit): the norm that follows adds a token's ``top``
+//                      parts in the order of j.
+//                  Any sizes, every multiply-add in IEEE 32-bit.
+#include "common.h"
+
+__device__ __forceinline__ void wave_argmax(float& v, int& i) {
+    for (int o = 32; o >= 1; o >>= 1) {
+        const float ov = __shfl_xor(v, o, 64);
+        const int oi = __shfl_xor(i, o, 64);
+        if (ov > v || (ov == v && oi >= 0 && (i < 0 || oi < i))) { v = ov; i = oi; }
+    }
+}
+
+// One wave per token.  Marks in the score table: -2 not (or no longer) a candidate.
+__global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, int* __restrict__ ids,
+                                                       float* __restrict__ weights, int E, int G, int keep, int top) {
+    extern __shared__ float sc[];          // E scores, G group scores
+    float* gs = sc + E;
+    const long t = blockIdx.x;
+    const int lane = threadIdx.x;
+    const float* z = logits + t * E;
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) {
+        const float ex = expf(z[e] - mx);
+        sc[e] = ex;
+        sum += ex;
+    }
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += 64) {
+        float v = sc[e] / sum;
+        if (!(v == v)) v = 0.f;            // (a row of garbage still gets experts inside the table)
+        sc[e] = v;
+    }
+    __syncthreads();
+    if (keep < G) {
+        const int per = E / G;
+        for (int g = lane; g < G; g += 64) {
+            float m = -1.f;
+            for (int e = g * per; e < (g + 1) * per; ++e) m = fmaxf(m, sc[e]);
+            gs[g] = m;
+        }
+        __syncthreads();
+        for (int r = 0; r < keep; ++r) {
+            float bv = -1.f;
+            int bi = -1;
+            for (int g = lane; g < G; g += 64)
+                if (gs[g] > bv) { bv = gs[g]; bi = g; }
+            wave_argmax(bv, bi);
+            if (lane == 0 && bi >= 0) gs[bi] = -3.f;       // kept
+            __syncthreads();
+        }
+        for (int e = lane; e < E; e += 64)
+            if (gs[e / per] != -3.f) sc[e] = -2.f;
+        __syncthreads();
+    }
+    for (int r = 0; r < top; ++r) {
+        float bv = -1.f;
+        int bi = -1;
+        for (int e = lane; e < E; e += 64)
+            if (sc[e] > bv) { bv = sc[e]; bi = e; }
+        wave_argmax(bv, bi);
+        if (lane == 0) {
+            ids[t * top + r] = bi >= 0 ? bi : 0;
+            weights[t * top + r] = bi >= 0 ? bv : 0.f;
+            if (bi >= 0) sc[bi] = -2.f;
+        }
+        __syncthreads();
+    }
+}
+
+extern "C" int qe_moe_route(const float* logits, int* ids, float* weights, int T, int E, int G, int keep, int top,
+                            hipStream_t stream) {
+    QE_REQUIRE(T >= 0 && E > 0 && G > 0 && E % G == 0, "moe_route: %d experts in %d groups", E, G);
+    QE_REQUIRE(keep >= 1 && keep <= G && top >= 1 && top <= keep * (E / G), "moe_route: top %d of %d groups of %d", top, keep, E / G);
+    QE_REQUIRE((E + G) * sizeof(float) <= 60000, "moe_route: too many experts");
+    if (T == 0) return 0;
+    moe_route_kernel<<<T, 64, (E + G) * sizeof(float), stream>>>(logits, ids, weights, E, G, keep, top);
+    QE_LAUNCH_CHECK();
+    return 0;
+}
+
+// One block.  n = T * top pairs.
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ ids, int n, int E, int tile_rows,
+                                                        int* __restrict__ perm, int* __restrict__ tiles,
+                                                        int* __restrict__ n_tiles) {
+    extern __shared__ int sm[];
+    int* counts = sm;
+    int* start = sm + E;
+    int* cursor = sm + 2 * E;
+    const int tid = threadIdx.x;
+    for (int e = tid; e < E; e += blockDim.x) counts[e] = 0;
+    __syncthreads();
+    for (int i = tid; i < n; i += blockDim.x) atomicAdd(&counts[ids[i]], 1);
+    __syncthreads();
+    for (int e = tid; e < E; e += blockDim.x) {
+        int off = 0, tb = 0;
+        for (int j = 0; j < e; ++j) {
+            off += counts[j];
+            tb += (counts[j] + tile_rows - 1) / tile_rows;
+        }
+        start[e] = off;
+        cursor[e] = off;
+        const int c = counts[e];
+        const int mine = (c + tile_rows - 1) / tile_rows;
+        for (int k = 0; k < mine; ++k) {
+            tiles[3 * (tb + k)] = e;
+            tiles[3 * (tb + k) + 1] = off + k * tile_rows;
+            tiles[3 * (tb + k) + 2] = c - k * tile_rows < tile_rows ? c - k * tile_rows : tile_rows;
+        }
+        if (e == E - 1) n_tiles[0] = tb + mine;
+    }
+    __syncthreads();
+    for (int i = tid; i < n; i += blockDim.x) perm[atomicAdd(&cursor[ids[i]], 1)] = i;
+}
+
+extern "C" int qe_moe_sort(const int* ids, int n, int E, int tile_rows, int* perm, int* tiles, int* n_tiles,
+                           int max_tiles, hipStream_t stream) {
+    QE_REQUIRE(n >= 0 && E > 0 && tile_rows > 0, "moe_sort: bad sizes");
+    QE_REQUIRE(max_tiles >= (n + tile_rows - 1) / tile_rows + (E < n ? E : n), "moe_sort: %d tiles may not be enough", max_tiles);
+    QE_REQUIRE(3 * E * sizeof(int) <= 60000, "moe_sort: too many experts");
+    moe_sort_kernel<<<1, 1024, 3 * E * sizeof(int), stream>>>(ids, n, E, tile_rows, perm, tiles, n_tiles);
+    QE_LAUNCH_CHECK();
+    return 0;
+}
+
+#define MT 64
+#define MK 16
+
+template <typename TA, typename TW, bool DUAL>
+__global__ __launch_bounds__(256) void moe_gemm_kernel(
+    const TA* __restrict__ x, const int* __restrict__ perm, int top, const TW* __restrict__ w, void* __restrict__ out_,
+    const float* __restrict__ weights, const int* __restrict__ tiles, const int* __restrict__ n_tiles, int T, int N,
+    int K, float limit, float slope) {
+    if ((int)blockIdx.y >= n_tiles[0]) return;
+    __shared__ float xs[MK][MT + 4];
+    __shared__ float ws[MK][MT + 4];
+    __shared__ float wu[DUAL ? MK : 1][MT + 4];
+    __shared__ int src[MT];              // the row of x behind each row of the tile, -1 beyond its rows
+    const int tid = threadIdx.x;
+    const int e = tiles[3 * blockIdx.y], r0 = tiles[3 * blockIdx.y + 1], rows = tiles[3 * blockIdx.y + 2];
+    const int n0 = blockIdx.x * MT;
+    if (tid < MT) src[tid] = tid < rows ? (DUAL ? perm[r0 + tid] / top : r0 + tid) : -1;
+    __syncthreads();
+    const int lr = tid >> 2;
+    const int lk = (tid & 3) * 4;
+    const int ty = tid >> 4, tx = tid & 15;
+    const TW* we = w + (long)e * (DUAL ? 2 : 1) * N * K;
+    const int xrow = src[lr];
+    float acc[4][4], acu[DUAL ? 4 : 1][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            acc[i][j] = 0.f;
+            if (DUAL) acu[i][j] = 0.f;
+        }
+    for (int k0 = 0; k0 < K; k0 += MK) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int k = k0 + lk + i;
+            const int n = n0 + lr;
+            xs[lk + i][lr] = (xrow >= 0 && k < K) ? Elem<TA>::load(x + (long)xrow * K + k) : 0.f;
+            ws[lk + i][lr] = (n < N && k < K) ? Elem<TW>::load(we + (long)n * K + k) : 0.f;
+            if (DUAL) wu[lk + i][lr] = (n < N && k < K) ? Elem<TW>::load(we + (long)(N + n) * K + k) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < MK; ++kk) {
+            float a[4], b[4], c[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = xs[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                b[j] = ws[kk][tx * 4 + j];
+                if (DUAL) c[j] = wu[kk][tx * 4 + j];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+                    if (DUAL) acu[i][j] = fmaf(a[i], c[j], acu[i][j]);
+                }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = ty * 4 + i;
+        if (m >= rows) continue;
+        if (DUAL) {
+            TA* o = (TA*)out_ + (long)(r0 + m) * N;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int n = n0 + tx * 4 + j;
+                if (n >= N) continue;
+                const float g = fminf(acc[i][j], limit);
+                const float u = fminf(fmaxf(acu[i][j], -limit), limit);
+                Elem<TA>::store(o + n, g / (1.f + expf(-slope * g)) * (u + 1.f));
+            }
+        } else {
+            const int pair = perm[r0 + m];
+            const float wgt = weights[pair];
+            float* o = (float*)out_ + ((long)(pair % top) * T + pair / top) * N;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int n = n0 + tx * 4 + j;
+                if (n < N) o[n] = wgt * acc[i][j];
+            }
+        }
+    }
+}
+
+// dual != 0: x [T, K] rows of the pairs' tokens, w [E, 2 N, K], out [T * top, N] in x's type at the sorted rows.
+// dual == 0: x [T * top, K] sorted rows, w [E, N, K], out float [top, T, N].
+extern "C" int qe_moe_gemm(const void* x, const int* perm, int top, const void* w, void* out, const float* weights,
+                           const int* tiles, const int* n_tiles, int max_tiles, int T, int N, int K, float limit,
+                           float slope, int dual, int dt_a, int dt_w, hipStream_t stream) {
+    QE_REQUIRE(T >= 0 && N > 0 && K > 0 && top > 0 && max_tiles >= 0 && max_tiles <= 65535, "moe_gemm: bad sizes");
+    if (T == 0 || max_tiles == 0) return 0;
+    dim3 grid(qe_cdiv(N, MT), max_tiles);
+#define QE_MG(TA_, TW_)                                                                                              \
+    do {                                                                                                             \
+        if (dual) moe_gemm_kernel<TA_, TW_, true><<<grid, 256, 0, stream>>>((const TA_*)x, perm, top, (const TW_*)w, out, weights, tiles, n_tiles, T, N, K, limit, slope); \
+        else moe_gemm_kernel<TA_, TW_, false><<<grid, 256, 0, stream>>>((const TA_*)x, perm, top, (const TW_*)w, out, weights, tiles, n_tiles, T, N, K, limit, slope);     \
+    } while (0)
+    if (dt_a == QE_F32 && dt_w == QE_F32) QE_MG(float, float);
+    else if (dt_a == QE_BF16 && dt_w == QE_BF16) QE_MG(bf16_t, bf16_t);
+    else QE_REQUIRE(false, "moe_gemm: no kernel for element types x=%d w=%d", dt_a, dt_w);
+#undef QE_MG
+    QE_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int qe_moe_tile_rows() { return MT; }

@@ -1,0 +1,98 @@
+// Norm after the residual sum, with one gain for all coordinates, on the 32-bit stream:
+//   z = alpha * x + (delta_0 + delta_1 + ...);   x <- g * z * rsqrt(mean(z^2) + eps)
+// and, if asked for, a copy of the new x in the activation type (what the next products read).
+// delta holds n_delta tensors [T, H] one after the other (one branch output, or partial products
+// of a matrix product, or the weighted outputs of a token's experts); they are added in ascending
+// order, so a row's sum does not depend on what else is in the batch.  All arithmetic in 32-bit.
+//
+// And the activation of the dense feed-forward that goes with this norm:
+//   act(z) = a z / rms(z) + b z^2 / rms(z^2) + c z^3 / rms(z^3) + e     per row, powers element by element
+#include "common.h"
+
+// One block per row.  The first pass writes z over x (every thread its own elements), the second
+// reads it back.
+template <typename TA, typename TD>
+__global__ void postnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta, int n_delta, long delta_stride,
+                                float alpha, const float* __restrict__ gain, float eps, TA* __restrict__ act,
+                                int H) {
+    __shared__ float red[16];
+    const long r = blockIdx.x;
+    float* xr = x + r * H;
+    const TD* dr = delta ? delta + r * H : nullptr;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float d = 0.f;
+        if (dr) {
+            d = Elem<TD>::load(dr + c);
+            for (int s = 1; s < n_delta; ++s) d += Elem<TD>::load(dr + s * delta_stride + c);
+        }
+        const float z = fmaf(alpha, xr[c], d);
+        xr[c] = z;
+        ss += z * z;
+    }
+    ss = block_sum(ss, red);
+    const float f = rsqrtf(ss / (float)H + eps) * gain[0];
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        const float v = xr[c] * f;
+        xr[c] = v;
+        if (act) Elem<TA>::store(act + r * H + c, v);
+    }
+}
+
+// dt_d: element type of delta; dt_a: of the copy (act may be null: no copy)
+extern "C" int qe_postnorm(float* x, const void* delta, int n_delta, int dt_d, float alpha, const float* gain,
+                           float eps, void* act, int dt_a, int T, int H, hipStream_t stream) {
+    QE_REQUIRE(T >= 0 && H > 0, "postnorm: bad sizes T=%d H=%d", T, H);
+    QE_REQUIRE(!delta || n_delta >= 1, "postnorm: %d delta tensors", n_delta);
+    if (T == 0) return 0;
+    const long stride = (long)T * H;
+    const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
+#define QE_PN(TA_, TD_) postnorm_kernel<TA_, TD_><<<T, threads, 0, stream>>>(x, (const TD_*)delta, n_delta, stride, alpha, gain, eps, (TA_*)act, H)
+    const int dd = delta ? dt_d : QE_F32;
+    if (dt_a == QE_F32 && dd == QE_F32) QE_PN(float, float);
+    else if (dt_a == QE_BF16 && dd == QE_F32) QE_PN(bf16_t, float);
+    else if (dt_a == QE_BF16 && dd == QE_BF16) QE_PN(bf16_t, bf16_t);
+    else QE_REQUIRE(false, "postnorm: no kernel for copy type %d with delta type %d", dt_a, dt_d);
+#undef QE_PN
+    QE_LAUNCH_CHECK();
+    return 0;
+}
+
+// One block per row of z [T, F] (32-bit); coef = (a, b, c, e).
+template <typename TA>
+__global__ void polynorm_kernel(const float* __restrict__ z, const float* __restrict__ coef, float eps,
+                                TA* __restrict__ out, int F) {
+    __shared__ float red[16];
+    const long r = blockIdx.x;
+    const float* zr = z + r * F;
+    float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    for (int c = threadIdx.x; c < F; c += blockDim.x) {
+        const float v = zr[c], v2 = v * v, v3 = v2 * v;
+        s1 += v2;
+        s2 += v2 * v2;
+        s3 += v3 * v3;
+    }
+    s1 = block_sum(s1, red);
+    s2 = block_sum(s2, red);
+    s3 = block_sum(s3, red);
+    const float a = coef[0] * rsqrtf(s1 / (float)F + eps);
+    const float b = coef[1] * rsqrtf(s2 / (float)F + eps);
+    const float cc = coef[2] * rsqrtf(s3 / (float)F + eps);
+    const float e = coef[3];
+    for (int c = threadIdx.x; c < F; c += blockDim.x) {
+        const float v = zr[c], v2 = v * v;
+        Elem<TA>::store(out + r * F + c, fmaf(a, v, fmaf(b, v2, fmaf(cc, v2 * v, e))));
+    }
+}
+
+extern "C" int qe_polynorm(const float* z, const float* coef, float eps, void* out, int dt_a, int T, int F,
+                           hipStream_t stream) {
+    QE_REQUIRE(T >= 0 && F > 0, "polynorm: bad sizes T=%d F=%d", T, F);
+    if (T == 0) return 0;
+    const int threads = F >= 2048 ? 512 : (F >= 512 ? 256 : 64);
+    if (dt_a == QE_F32) polynorm_kernel<float><<<T, threads, 0, stream>>>(z, coef, eps, (float*)out, F);
+    else if (dt_a == QE_BF16) polynorm_kernel<bf16_t><<<T, threads, 0, stream>>>(z, coef, eps, (bf16_t*)out, F);
+    else QE_REQUIRE(false, "polynorm: unknown output type %d", dt_a);
+    QE_LAUNCH_CHECK();
+    return 0;
+}

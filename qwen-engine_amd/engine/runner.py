@@ -117,7 +117,7 @@ class ModelRunner:
                 self.kv.append(None)
                 continue
             pages = self.cache.pools[self.plan.user_group[u]].num_pages
-            self.kv.append(torch.full((pages, 2, need.num_kv_heads, page_size, need.head_dim),
+            self.kv.append(torch.full((pages, need.planes, need.num_kv_heads, page_size, need.head_dim),
                                       float("nan") if self.debug_poison else 0.0, dtype=dt, device=dev))
         self.state: List[Optional[torch.Tensor]] = []
         for need in self.plan.user_state:

@@ -79,6 +79,17 @@ def load_library():
         "qe_argmax": [vp, vp, i32, i32, vp, i64, vp],
         "qe_argmax_static": [vp, vp, i32, i32, vp],
         "qe_sample": [vp, vp, vp, vp, i32, i32, vp],
+        "qe_postnorm": [vp, vp, i32, i32, f32, vp, f32, vp, i32, i32, i32, vp],
+        "qe_polynorm": [vp, vp, f32, vp, i32, i32, i32, vp],
+        "qe_short_conv": [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp],
+        "qe_latent_kv_store": [vp, vp, f32, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp],
+        "qe_latent_q_rotate": [vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, i32, vp],
+        "qe_latent_attention": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, vp],
+        "qe_gemm_heads": [vp, i64, i64, vp, vp, i64, i64, vp, i32, i32, i32, i32, i32, i32, vp],
+        "qe_moe_route": [vp, vp, vp, i32, i32, i32, i32, i32, vp],
+        "qe_moe_sort": [vp, i32, i32, i32, vp, vp, vp, i32, vp],
+        "qe_moe_gemm": [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, f32, i32, i32, i32, vp],
+        "qe_moe_tile_rows": [],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
@@ -808,3 +819,197 @@ def mfma_probe(blocks: int = 512, iters: int = 20000, device="cuda:0") -> float:
         end.synchronize()
         best = max(best, flops.value / (start.elapsed_time(end) * 1e-3))
     return best
+
+
+# ---- norm after the residual sum, the short convolution, the polynomial activation ------------------
+def postnorm(x: torch.Tensor, delta: Optional[torch.Tensor], alpha: float, gain: torch.Tensor, eps: float,
+             act_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """x <- gain * z / sqrt(mean(z^2) + eps) with z = alpha * x + delta, on the 32-bit stream x [T, H], in
+    place.  delta: None, [T, H] (bfloat16 or float32) or float32 [S, T, H], added in the order of S.  gain:
+    float32 [1].  With ``act_dtype`` bfloat16 a copy of the new x in that type is returned (what the next
+    products read); with float32 or None, nothing (the stream itself is read)."""
+    lib = load_library()
+    _need(x, "x", torch.float32, (None, None))
+    T, H = x.shape
+    _need(gain, "gain", torch.float32, (1,), x.device)
+    n_delta, dt_d = 0, F32
+    if delta is not None:
+        if delta.dim() == 3:
+            _need(delta, "delta", torch.float32, (None, T, H), x.device)
+            n_delta = delta.shape[0]
+        else:
+            _need(delta, "delta", _ACT, (T, H), x.device)
+            n_delta, dt_d = 1, _DT[delta.dtype]
+    act = None
+    if act_dtype == torch.bfloat16:
+        act = torch.empty((T, H), dtype=torch.bfloat16, device=x.device)
+    _check(lib.qe_postnorm(x.data_ptr(), _ptr(delta), n_delta, dt_d, float(alpha), gain.data_ptr(), float(eps),
+                           _ptr(act), BF16 if act is not None else F32, T, H, _stream()), "postnorm")
+    return act
+
+
+def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """a z / rms(z) + b z^2 / rms(z^2) + c z^3 / rms(z^3) + e per row of z (float32 [T, F]), rms(v) =
+    sqrt(mean(v^2) + eps), coef = (a, b, c, e) float32 [4]; all in 32-bit, one rounding at the store."""
+    lib = load_library()
+    _need(z, "z", torch.float32, (None, None))
+    T, Fd = z.shape
+    _need(coef, "coef", torch.float32, (4,), z.device)
+    out = torch.empty((T, Fd), dtype=out_dtype, device=z.device)
+    _check(lib.qe_polynorm(z.data_ptr(), coef.data_ptr(), float(eps), out.data_ptr(), _DT[out_dtype], T, Fd, _stream()),
+           "polynorm")
+    return out
+
+
+def short_conv(x: torch.Tensor, w: torch.Tensor, state: Optional[torch.Tensor], tok_seq: torch.Tensor,
+               out_dtype: torch.dtype, update: bool = True) -> torch.Tensor:
+    """out_t = x_t + sum_k w[:, taps - 1 - k] x_(t - k) along each request's tokens, x the 32-bit stream
+    [T, H], w float32 [H, taps].  What lies before a request's rows in this step comes from state
+    (float32 [slots, taps - 1, H], row tok_seq[t]: the request's last taps - 1 inputs), which then takes
+    the step's last inputs (``update``).  The rows of a request are consecutive."""
+    lib = load_library()
+    _need(x, "x", torch.float32, (None, None))
+    T, H = x.shape
+    _need(w, "w", torch.float32, (H, None), x.device)
+    taps = w.shape[1]
+    _need(tok_seq, "tok_seq", torch.int32, (T,), x.device)
+    if taps > 1:
+        if state is None:
+            raise KernelError("short_conv: no state")
+        _need(state, "state", torch.float32, (None, taps - 1, H), x.device)
+    out = torch.empty((T, H), dtype=out_dtype, device=x.device)
+    _check(lib.qe_short_conv(x.data_ptr(), w.data_ptr(), _ptr(state), tok_seq.data_ptr(), out.data_ptr(),
+                             _DT[out_dtype], T, H, taps, int(update), _stream()), "short_conv")
+    return out
+
+
+# ---- attention over one cached latent per token --------------------------------------------------------
+def latent_kv_store(kv: torch.Tensor, weight: torch.Tensor, eps: float, positions: torch.Tensor,
+                    inv_freq: torch.Tensor, slots: torch.Tensor, cache: torch.Tensor) -> None:
+    """kv float32 [T, R + Dr] (R = weight's length): the first R normed (weight * u / rms(u)), the last Dr
+    turned in neighbouring pairs by positions * inv_freq (float32 [n], 2 n <= Dr; the rest passes), into
+    the row slots[t] of cache [pages, 1, 1, P, R + Dr] (negative slot: nowhere)."""
+    lib = load_library()
+    _need(kv, "kv", torch.float32, (None, None))
+    T, D = kv.shape
+    dev = kv.device
+    _need(weight, "weight", torch.float32, (None,), dev)
+    R = weight.shape[0]
+    _need(cache, "cache", _ACT, (None, 1, 1, None, D), dev)
+    _need(positions, "positions", torch.int32, (T,), dev)
+    _need(slots, "slots", torch.int32, (T,), dev)
+    _need(inv_freq, "inv_freq", torch.float32, (None,), dev)
+    _check(lib.qe_latent_kv_store(kv.data_ptr(), weight.data_ptr(), float(eps), positions.data_ptr(),
+                                  inv_freq.data_ptr(), 2 * inv_freq.shape[0], slots.data_ptr(), cache.data_ptr(),
+                                  _DT[cache.dtype], T, R, D - R, _stream()), "latent_kv_store")
+
+
+def latent_q_rotate(q: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, qp: torch.Tensor,
+                    dim: int) -> None:
+    """q [T, H, dim + Dr] -> the last Dr of each head, turned as in latent_kv_store, into the last Dr of
+    qp [T, H, R + Dr]."""
+    lib = load_library()
+    _need(q, "q", _ACT, (None, None, None))
+    T, H, Dq = q.shape
+    Dr = Dq - int(dim)
+    _need(qp, "qp", q.dtype, (T, H, None), q.device)
+    R = qp.shape[2] - Dr
+    if Dr < 0 or R <= 0:
+        raise KernelError("latent_q_rotate: sizes do not fit")
+    _need(positions, "positions", torch.int32, (T,), q.device)
+    _need(inv_freq, "inv_freq", torch.float32, (None,), q.device)
+    _check(lib.qe_latent_q_rotate(q.data_ptr(), positions.data_ptr(), inv_freq.data_ptr(), 2 * inv_freq.shape[0],
+                                  qp.data_ptr(), _DT[q.dtype], T, H, int(dim), Dr, R, _stream()), "latent_q_rotate")
+
+
+def latent_attention(qp: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
+                     block_table: torch.Tensor, latent: int, scale: float) -> torch.Tensor:
+    """qp [T, H, R + Dr], cache [pages, 1, 1, P, R + Dr]: per (token, head) softmax(scale * qp . rows) . rows[:R]
+    over the rows at positions 0 .. p of request tok_seq[t] -> [T, H, R].  32-bit scores and weights."""
+    lib = load_library()
+    _need(qp, "qp", _ACT, (None, None, None))
+    T, H, D = qp.shape
+    dev = qp.device
+    R = int(latent)
+    _need(cache, "cache", qp.dtype, (None, 1, 1, None, D), dev)
+    P = cache.shape[3]
+    _need(positions, "positions", torch.int32, (T,), dev)
+    _need(tok_seq, "tok_seq", torch.int32, (T,), dev)
+    _need(block_table, "block_table", torch.int32, (None, None), dev)
+    out = torch.empty((T, H, R), dtype=qp.dtype, device=dev)
+    _check(lib.qe_latent_attention(qp.data_ptr(), out.data_ptr(), cache.data_ptr(), positions.data_ptr(),
+                                   tok_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, H, R, D - R, P,
+                                   float(scale), _DT[qp.dtype], _stream()), "latent_attention")
+    return out
+
+
+def gemm_heads(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t, h, :N] = w[h] x[t, h, :K] for w [H, N, K]; x [T, H, >= K] and out [T, H, >= N] (the product reads
+    the first K and writes the first N numbers of each head).  gate [T, H * N]: the result times
+    sigmoid(gate)."""
+    lib = load_library()
+    _need(w, "w", _ACT, (None, None, None))
+    H, N, K = w.shape
+    _need(x, "x", _ACT, (None, H, None))
+    T = x.shape[0]
+    _need(out, "out", x.dtype, (T, H, None), x.device)
+    if x.shape[2] < K or out.shape[2] < N:
+        raise KernelError("gemm_heads: heads narrower than the product")
+    if x.dtype == torch.float32 and w.dtype != torch.float32:
+        raise KernelError("gemm_heads: 32-bit activations need 32-bit weights")
+    if gate is not None:
+        _need(gate, "gate", x.dtype, (T, H * N), x.device)
+    _check(lib.qe_gemm_heads(x.data_ptr(), H * x.shape[2], x.shape[2], w.data_ptr(), out.data_ptr(),
+                             H * out.shape[2], out.shape[2], _ptr(gate), T, H, N, K, _DT[x.dtype], _DT[w.dtype],
+                             _stream()), "gemm_heads")
+    return out
+
+
+# ---- mixture of experts -----------------------------------------------------------------------------------
+def moe_route(logits: torch.Tensor, groups: int, keep: int, top: int):
+    """logits float32 [T, E] -> (ids int32 [T, top], weights float32 [T, top]): softmax over all experts,
+    the ``keep`` best of ``groups`` equal groups of neighbours (a group's score is its largest), the ``top``
+    largest scores among them, as they are."""
+    lib = load_library()
+    _need(logits, "logits", torch.float32, (None, None))
+    T, E = logits.shape
+    ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    _check(lib.qe_moe_route(logits.data_ptr(), ids.data_ptr(), weights.data_ptr(), T, E, int(groups), int(keep),
+                            int(top), _stream()), "moe_route")
+    return ids, weights
+
+
+def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor,
+                w_down: torch.Tensor, limit: float, slope: float) -> torch.Tensor:
+    """The chosen experts' outputs, weighted: float32 [top, T, H], the parts of a token's sum in the order of
+    its choices.  x [T, K]; w_gate_up [E, 2 F, K] (gate rows, then up rows); w_down [E, H, F].  An expert:
+    g = min(gate x, limit), u = clamp(up x, -limit, limit), down (g sigmoid(slope g) (u + 1))."""
+    lib = load_library()
+    _need(x, "x", _ACT, (None, None))
+    T, K = x.shape
+    dev = x.device
+    _need(ids, "ids", torch.int32, (T, None), dev)
+    top = ids.shape[1]
+    _need(weights, "weights", torch.float32, (T, top), dev)
+    _need(w_gate_up, "w_gate_up", x.dtype, (None, None, K), dev)
+    E, F2 = w_gate_up.shape[0], w_gate_up.shape[1]
+    Fd = F2 // 2
+    _need(w_down, "w_down", x.dtype, (E, None, Fd), dev)
+    Hout = w_down.shape[1]
+    n = T * top
+    tile_rows = lib.qe_moe_tile_rows()
+    max_tiles = (n + tile_rows - 1) // tile_rows + min(E, n)
+    meta = torch.empty(n + 3 * max_tiles + 1, dtype=torch.int32, device=dev)
+    perm, tiles, n_tiles = meta[:n], meta[n:n + 3 * max_tiles], meta[n + 3 * max_tiles:]
+    _check(lib.qe_moe_sort(ids.data_ptr(), n, E, tile_rows, perm.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr(),
+                           max_tiles, _stream()), "moe_sort")
+    a = torch.empty((n, Fd), dtype=x.dtype, device=dev)
+    _check(lib.qe_moe_gemm(x.data_ptr(), perm.data_ptr(), top, w_gate_up.data_ptr(), a.data_ptr(), None,
+                           tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, T, Fd, K, float(limit), float(slope), 1,
+                           _DT[x.dtype], _DT[w_gate_up.dtype], _stream()), "moe_gemm (gate, up)")
+    parts = torch.empty((top, T, Hout), dtype=torch.float32, device=dev)
+    _check(lib.qe_moe_gemm(a.data_ptr(), perm.data_ptr(), top, w_down.data_ptr(), parts.data_ptr(), weights.data_ptr(),
+                           tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, T, Hout, Fd, 0.0, 0.0, 0,
+                           _DT[x.dtype], _DT[w_down.dtype], _stream()), "moe_gemm (down)")
+    return parts

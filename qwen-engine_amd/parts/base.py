@@ -67,6 +67,20 @@ class TensorInfo(NamedTuple):
     shape: Tuple[int, ...]
     init: str = "normal"   # "normal": N(0, std); "ones": norm weight; "zeros": bias
     role: str = "matrix"   # "matrix" keeps the stored element type in bfloat16 mode; "vector" is held in 32-bit
+    optional: bool = False  # a folder may lack it: the part then finds no such name among its tensors
+
+
+def join_name(prefix: str, rel: str) -> str:
+    """A tensor's checkpoint name from its owner's name and its name inside the owner; a part that is one
+    tensor names it "" and the tensor carries the owner's name."""
+    if not prefix:
+        return rel
+    return f"{prefix}.{rel}" if rel else prefix
+
+
+def named_tensors(tensors, prefix: str, names):
+    """{rel: tensor} for the relative names ``names`` of the owner ``prefix`` that ``tensors`` holds."""
+    return {rel: tensors[join_name(prefix, rel)] for rel in names if join_name(prefix, rel) in tensors}
 
 
 def sub_tensors(tensors, prefix: str):

@@ -8,7 +8,7 @@ from typing import Dict, Optional
 
 import torch
 
-from .base import CacheBinding, Runtime, Stream, StreamInput, TensorInfo, sub_tensors
+from .base import CacheBinding, Runtime, Stream, StreamInput, TensorInfo, join_name, named_tensors, sub_tensors
 from ..kernels import ops
 from .registry import build_part, part_class, register_part
 
@@ -86,4 +86,106 @@ class PreNormBlock:
         return norm.forward(stream.h, ctx.rt, delta=delta)
 
 
+class PostNormBlock:
+    """x <- mixer_norm(alpha x + mixer(conv(x))); x <- ffn_norm(alpha x + ffn(x)).  The stream x stays
+    32-bit and normed; each norm forms the sum, norms it in place and hands the next part a copy in the
+    activation type.  The convolution in front of the mixer keeps a request's last inputs in the block's
+    state slot; the mixer keeps its cache: one cache user with both."""
+
+    def __init__(self, spec, hidden_size: int):
+        self.spec = spec
+        self.hidden = int(hidden_size)
+        self.alpha = float(spec.alpha)
+        self.mixer_norm = build_part(spec.mixer_norm, hidden_size)
+        self.mixer = build_part(spec.mixer, hidden_size)
+        self.ffn = build_part(spec.ffn, hidden_size) if spec.ffn is not None else None
+        # without a feed-forward the second norm is there only if the folder holds its tensor
+        self.ffn_norm = build_part(spec.ffn_norm or spec.mixer_norm, hidden_size)
+        self.has_ffn_norm = spec.ffn is not None
+        self.conv = build_part(spec.conv, hidden_size) if spec.conv is not None else None
+
+    def parts(self):
+        return tuple(p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn, self.conv) if p is not None)
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(p, "graph_safe", True) for p in self.parts())
+
+    @property
+    def graph_safe_with_state(self) -> bool:
+        return all(getattr(p, "graph_safe", False) is True for p in (self.mixer, self.conv) if p is not None)
+
+    @staticmethod
+    def _named(spec):
+        """(checkpoint name, part spec, optional) of the block's parts."""
+        n_norm1, n_mix, n_norm2, n_ffn, n_conv = spec.names
+        out = [(n_norm1, spec.mixer_norm, False), (n_mix, spec.mixer, False)]
+        if spec.ffn is not None:
+            out += [(n_norm2, spec.ffn_norm or spec.mixer_norm, False), (n_ffn, spec.ffn, False)]
+        else:
+            out += [(n_norm2, spec.ffn_norm or spec.mixer_norm, True)]
+        if spec.conv is not None:
+            out.append((n_conv, spec.conv, False))
+        return out
+
+    @staticmethod
+    def cache_needs(spec, hidden: int):
+        cls = part_class(spec.mixer.kind)
+        kv = cls.cache_need(spec.mixer) if hasattr(cls, "cache_need") else None
+        state = part_class(spec.conv.kind).state_need(spec.conv, hidden) if spec.conv is not None else None
+        mixer_state = cls.state_need(spec.mixer, hidden) if hasattr(cls, "state_need") else None
+        if mixer_state is not None:
+            raise ValueError("a post-norm block's state slot belongs to its convolution: the mixer cannot ask for one too")
+        return [(kv, state)]
+
+    @staticmethod
+    def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
+        out: Dict[str, TensorInfo] = {}
+        for name, sub, optional in PostNormBlock._named(spec):
+            for rel, info in part_class(sub.kind).expected_tensors(sub, hidden).items():
+                out[join_name(name, rel)] = info._replace(optional=True) if optional else info
+        return out
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        n_norm1, n_mix, n_norm2, n_ffn, n_conv = self.spec.names
+        for name, part in ((n_norm1, self.mixer_norm), (n_mix, self.mixer), (n_norm2, self.ffn_norm),
+                           (n_ffn, self.ffn), (n_conv, self.conv)):
+            if part is None:
+                continue
+            names = type(part).expected_tensors(self._spec_of(part), self.hidden)
+            held = named_tensors(tensors, name, names)
+            if part is self.ffn_norm and self.ffn is None:
+                self.has_ffn_norm = len(held) == len(names)
+                if not self.has_ffn_norm:
+                    continue
+            part.load(held, rt)
+
+    def _spec_of(self, part):
+        s = self.spec
+        return {id(self.mixer_norm): s.mixer_norm, id(self.mixer): s.mixer, id(self.ffn_norm): s.ffn_norm or s.mixer_norm,
+                id(self.ffn): s.ffn, id(self.conv): s.conv}[id(part)]
+
+    def forward(self, h, pending: Optional[torch.Tensor], ctx, bindings):
+        """h: the 32-bit stream (a tensor, or a Stream).  pending: a branch output that a block of another
+        kind before this one left to be added.  Returns None: nothing is left to add."""
+        x = h.h if isinstance(h, Stream) else h
+        rt = ctx.rt
+        if pending is not None:
+            ops.residual_add(x, pending)
+        binding = bindings[0]
+        if self.conv is not None:
+            xin = self.conv.forward(x, ctx, binding.state)
+        else:
+            xin = x if rt.dtype == torch.float32 else x.to(rt.dtype)
+        y = self.mixer.forward(xin, ctx, binding)
+        xa = self.mixer_norm.after_sum(x, y, self.alpha, rt)
+        if self.ffn is not None:
+            y = self.ffn.forward(x if xa is None else xa, ctx)
+            self.ffn_norm.after_sum(x, y, self.alpha, rt)
+        elif self.has_ffn_norm:
+            self.ffn_norm.after_sum(x, None, self.alpha, rt)
+        return None
+
+
 register_part("prenorm_block", PreNormBlock)
+register_part("postnorm_block", PostNormBlock)

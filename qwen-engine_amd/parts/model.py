@@ -10,7 +10,7 @@ import torch
 from ..cache.plan import CachePlan, plan_cache
 from ..config.spec import ModelSpec
 from ..kernels import ops
-from .base import CacheBinding, Runtime, Stream, TensorInfo, sub_tensors
+from .base import CacheBinding, Runtime, Stream, TensorInfo, join_name, named_tensors, sub_tensors
 from .registry import build_part, part_class
 
 
@@ -19,11 +19,11 @@ def expected_tensors(spec: ModelSpec) -> Dict[str, TensorInfo]:
     out: Dict[str, TensorInfo] = {spec.embed_name: TensorInfo((spec.vocab_size, spec.hidden_size), "normal", "matrix")}
     for layer in spec.layers:
         for rel, info in part_class(layer.kind).expected_tensors(layer, spec.hidden_size).items():
-            out[f"{layer.prefix}.{rel}"] = info
+            out[join_name(layer.prefix, rel)] = info
     norm_rel = part_class(spec.final_norm.kind).expected_tensors(spec.final_norm, spec.hidden_size)
     base = spec.final_norm_name[:-len(".weight")] if spec.final_norm_name.endswith(".weight") else spec.final_norm_name
     for rel, info in norm_rel.items():
-        out[f"{base}.{rel}"] = info
+        out[join_name(base, rel)] = info
     if not spec.tie_head:
         out[spec.head_name] = TensorInfo((spec.vocab_size, spec.hidden_size), "normal", "matrix")
     for extra in (spec.stream_prologue, spec.logit_epilogue):
@@ -87,7 +87,8 @@ class DecoderModel:
         for layer, block in zip(spec.layers, self.blocks):
             block.load(sub_tensors(tensors, layer.prefix + "."), rt)
         base = spec.final_norm_name[:-len(".weight")] if spec.final_norm_name.endswith(".weight") else spec.final_norm_name
-        self.final_norm.load(sub_tensors(tensors, base + "."), rt)
+        names = part_class(spec.final_norm.kind).expected_tensors(spec.final_norm, spec.hidden_size)
+        self.final_norm.load(named_tensors(tensors, base, names), rt)
         self.head = self.embed if spec.tie_head else rt.place_matrix(tensors[spec.head_name])
         for part, part_spec in ((self.prologue, spec.stream_prologue), (self.epilogue, spec.logit_epilogue)):
             if part is not None:

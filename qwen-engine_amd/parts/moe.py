@@ -1,0 +1,92 @@
+"""Feed-forwards of a post-norm decoder: a dense one with a polynomial activation normed per power, and
+a routed mixture of small gated experts."""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import Runtime, TensorInfo
+from .registry import register_part
+
+
+class PolyNormMLP:
+    """down(a N(z) + b N(z^2) + c N(z^3) + e), z = up x, N(v) = v / sqrt(mean(v^2) + eps) per token.  The
+    up product leaves z in 32-bit; the activation is formed in 32-bit and rounded once."""
+    graph_safe = True
+
+    def __init__(self, spec, hidden_size: int):
+        self.hidden = int(hidden_size)
+        self.inter = int(spec.intermediate_size)
+        self.eps = float(spec.eps)
+        self.w_up = self.w_down = self.coef = None
+
+    @staticmethod
+    def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
+        i = spec.intermediate_size
+        return {"up": TensorInfo((i, hidden)), "down": TensorInfo((hidden, i)), "act": TensorInfo((4,), "ones", "vector")}
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        self.w_up = rt.place_matrix(tensors["up"])
+        self.w_down = rt.place_matrix(tensors["down"])
+        self.coef = rt.place_vector(tensors["act"])
+
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        z = ops.gemm(x, self.w_up, out_dtype=torch.float32)
+        a = ops.polynorm(z, self.coef, self.eps, ctx.rt.dtype)
+        splits = ops.gemm_branch_splits(a, self.w_down)
+        if splits:
+            return ops.gemm(a, self.w_down, epilogue=ops.EPI_PARTIAL, splits=splits)
+        return ops.gemm(a, self.w_down)
+
+
+class GroupedMoE:
+    """Router logits in 32-bit, softmax over all experts, the best groups of neighbouring experts, the
+    largest scores among them (``ops.moe_route``); then the chosen experts' two products over the
+    (token, choice) pairs grouped by expert on the device (``ops.moe_experts``).  The output is float32
+    [top, T, H]: a token's weighted expert outputs in the order of its choices, which the norm that
+    follows adds to the stream."""
+    graph_safe = True
+
+    def __init__(self, spec, hidden_size: int):
+        self.spec = spec
+        self.hidden = int(hidden_size)
+        self.e, self.top, self.inter = int(spec.num_experts), int(spec.top), int(spec.intermediate_size)
+        self.w_router = self.w_gate_up = self.w_down = None
+
+    @staticmethod
+    def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
+        f = spec.intermediate_size
+        t = {"router": TensorInfo((spec.num_experts, hidden))}
+        for e in range(spec.num_experts):
+            t[f"e{e}.gate"] = TensorInfo((f, hidden))
+            t[f"e{e}.up"] = TensorInfo((f, hidden))
+            t[f"e{e}.down"] = TensorInfo((hidden, f))
+        return t
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        self.w_router = rt.place_matrix(tensors["router"])
+        first = tensors["e0.gate"]
+        dt = torch.float32 if rt.dtype == torch.float32 or first.dtype == torch.float32 else torch.bfloat16
+        self.w_gate_up = torch.empty((self.e, 2 * self.inter, self.hidden), dtype=dt, device=rt.device)
+        self.w_down = torch.empty((self.e, self.hidden, self.inter), dtype=dt, device=rt.device)
+        for e in range(self.e):           # an expert at a time: the host never holds more
+            self.w_gate_up[e, :self.inter].copy_(tensors[f"e{e}.gate"])
+            self.w_gate_up[e, self.inter:].copy_(tensors[f"e{e}.up"])
+            self.w_down[e].copy_(tensors[f"e{e}.down"])
+
+    def active_weight_bytes(self, tokens: int) -> int:
+        """Bytes of expert weights that a step of ``tokens`` tokens reads at most."""
+        per = (self.w_gate_up[0].numel() + self.w_down[0].numel()) * self.w_down.element_size()
+        return min(self.e, tokens * self.top) * per + self.w_router.numel() * self.w_router.element_size()
+
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        s = self.spec
+        logits = ops.gemm(x, self.w_router, out_dtype=torch.float32)
+        ids, weights = ops.moe_route(logits, s.num_groups, s.keep_groups, s.top)
+        return ops.moe_experts(x, ids, weights, self.w_gate_up, self.w_down, s.limit, s.slope)
+
+
+register_part("polynorm_mlp", PolyNormMLP)
+register_part("grouped_moe", GroupedMoE)

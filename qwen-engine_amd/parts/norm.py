@@ -33,4 +33,33 @@ class RMSNorm:
         return ops.rmsnorm(h, self.weight, self.eps, rt.dtype, delta=delta, rows=rows)
 
 
+class ScalarRMSNorm:
+    """RMS norm with one gain for all coordinates (a tensor of no dimensions, named as the part itself).
+    ``forward`` is the norm interface of ``parts.base`` (the model's last norm, on the wanted rows);
+    ``after_sum`` is the norm of a post-norm block: x <- g * z / rms(z) with z = alpha * x + delta, on the
+    32-bit stream in place, returning the new x in the activation type where that is not 32-bit."""
+
+    def __init__(self, spec, size: int):
+        self.eps = float(spec.eps)
+        self.size = int(size)
+        self.gain: Optional[torch.Tensor] = None      # float32 [1]
+        self.weight: Optional[torch.Tensor] = None    # the gain, once per coordinate
+
+    @staticmethod
+    def expected_tensors(spec, size: int) -> Dict[str, TensorInfo]:
+        return {"": TensorInfo((), "ones", "vector")}
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        self.gain = rt.place_vector(tensors[""].reshape(1))
+        self.weight = self.gain.expand(self.size).contiguous()
+
+    def forward(self, h: torch.Tensor, rt: Runtime, delta: Optional[torch.Tensor] = None,
+                rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.rmsnorm(h, self.weight, self.eps, rt.dtype, delta=delta, rows=rows)
+
+    def after_sum(self, x: torch.Tensor, delta: Optional[torch.Tensor], alpha: float, rt: Runtime):
+        return ops.postnorm(x, delta, alpha, self.gain, self.eps, rt.dtype)
+
+
 register_part("rmsnorm", RMSNorm)
+register_part("rmsnorm_scalar", ScalarRMSNorm)

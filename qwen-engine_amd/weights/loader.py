@@ -89,10 +89,10 @@ def read_checked(folder: str, expected: Dict[str, TensorInfo], tied_head_name: s
         for name in f.keys():
             where[name] = len(handles) - 1
             shapes[name] = tuple(f.get_slice(name).get_shape())
-    missing = sorted(n for n in expected if n not in where)
+    missing = sorted(n for n in expected if n not in where and not getattr(expected[n], "optional", False))
     unexpected = sorted(n for n in where if n not in expected and n != tied_head_name)
     wrong = sorted((n, shapes[n], tuple(expected[n].shape)) for n in expected
                    if n in where and shapes[n] != tuple(expected[n].shape))
     if missing or unexpected or wrong:
         raise WeightError(folder, missing, unexpected, wrong)
-    return LazyTensors(handles, where, {name: name for name in expected})
+    return LazyTensors(handles, where, {name: name for name in expected if name in where})

@@ -32,6 +32,8 @@ def random_tensors(config, seed: int, dtype: torch.dtype = torch.bfloat16, std: 
     spec = config.to_model_spec()
     out: Dict[str, torch.Tensor] = {}
     for name, info in expected_tensors(spec).items():
+        if getattr(info, "optional", False):
+            continue
         g = _generator(seed, name)
         if info.init == "ones":
             t = torch.ones(info.shape, dtype=torch.float32)
