@@ -35,6 +35,10 @@ Other sizes and workloads (not what the default line reports):
                             recorded graph of repetitions over weights that do not fit the caches, and its rate
                             against the nominal and the measured peaks (the counterpart of the reference's
                             per-operator benchmarks, src/layers/ops/linear.py:204-249)
+  --design zarorax          another design beside the closest Qwen3 model of equal sizes (width, layers, heads, and a
+                            feed-forward as wide as the experts a token uses): prefill (one prompt of --prefill-tokens
+                            in one step) and decode (batch 1 and --batch at --context) of both, at the sizes of
+                            --design-sizes (small, medium); one JSON line of its own.  The default line is unchanged.
   --warmup-passes N         both: untimed passes over the workload with other tokens before the timed
                             one (default 2: the graphs are recorded there, a shape of steps when it is met
                             the second time, as in a server that has run for a while; 0 times the
@@ -90,6 +94,9 @@ def parse():
                     help="run steps of single new tokens beside a prompt portion as they come, not from a recorded graph")
     ap.add_argument("--requests", type=int, default=None, help="requests of the serving workloads")
     ap.add_argument("--kernels", action="store_true", help="time each kernel of a layer alone over a range of rows")
+    ap.add_argument("--design", default=None, choices=["zarorax"],
+                    help="measure this design beside the closest Qwen3 model of equal sizes instead of the default workload")
+    ap.add_argument("--design-sizes", default="small,medium", help="which of the design's sizes (small, medium), with commas")
     ap.add_argument("--warmup-passes", type=int, default=2,
                     help="serving workloads: untimed passes before the timed one (they record the decode graphs)")
     return ap.parse_args()
@@ -328,11 +335,129 @@ def kernel_sweep(args, cfg) -> int:
     return 0
 
 
+# Layer sizes for --design zarorax: (width, heads, unrotated, rotated, value, key/value latent, query latent,
+# dense ff, experts, chosen, groups, kept groups, expert ff)
+ZARORAX_SIZES = {
+    "small": dict(width=1024, heads=16, dim=64, rot_dim=32, vdim=64, kv_rank=256, q_rank=384, ff=3072,
+                  experts=32, top=4, groups=4, keep=2, expert_ff=768),
+    "medium": dict(width=2048, heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=768, ff=6144,
+                   experts=32, top=4, groups=4, keep=2, expert_ff=1024),
+}
+
+
+def zarorax_config(z, layers, vocab):
+    """A dense layer first, then mixtures, the two mixers in turn."""
+    def mixer(direct):
+        m = {"heads": z["heads"], "dim": z["dim"], "rot_dim": z["rot_dim"], "vdim": z["vdim"], "kv_rank": z["kv_rank"],
+             "scale": (z["dim"] + z["rot_dim"]) ** -0.5, "rot": {"base": 10000.0, "dims": z["rot_dim"]}}
+        if not direct:
+            m["q_rank"] = z["q_rank"]
+        return m
+    moe = {"kind": "moe", "expert": {"ff": z["expert_ff"], "limit": 7.0},
+           "router": {"experts": z["experts"], "top": z["top"], "groups": {"count": z["groups"], "keep": z["keep"]}}}
+    ls = []
+    for i in range(layers):
+        direct = i % 2 == 1
+        ls.append({"type": "latent_attention_2" if direct else "latent_attention", "mixer": mixer(direct),
+                   "mlp": {"kind": "dense", "ff": z["ff"]} if i == 0 else moe})
+    return {"architecture": "Zarorax", "vocab": vocab, "width": z["width"], "postln_alpha": 2.0, "norm": {"eps": 1e-5},
+            "canon": {"taps": 4}, "layers": ls}
+
+
+def design_compare(args) -> int:
+    """Prefill and decode of the Zarorax design beside the Qwen3 model of equal sizes, through the same step
+    function.  A "step" is one decode step; the line's value is the design's decode rate at --batch, first size."""
+    import torch
+    from qwen_engine_amd.config import config_from_dict
+    from qwen_engine_amd.engine import ModelRunner, StepEntry
+    from qwen_engine_amd.kernels import ops
+    from qwen_engine_amd.parts import DecoderModel, Runtime
+    from qwen_engine_amd.weights import random_tensors
+
+    dev = torch.device("cuda:0")
+    dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    P, V = args.block_size, 32768
+    layers = args.layers or 6
+    g = torch.Generator().manual_seed(args.seed + 1)
+
+    def measure(cfg):
+        t0 = time.time()
+        model = DecoderModel(cfg.to_model_spec())
+        model.load(random_tensors(cfg, args.seed, dtype=torch.bfloat16), Runtime(dev, dtype))
+        print(f"[bench] {cfg.architecture}: random weights in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+        res = {}
+        T = args.prefill_tokens
+        runner = ModelRunner(model, page_size=P, num_pages=(T + P - 1) // P + 1, max_requests=1)
+        toks = torch.randint(0, V, (T,), generator=g).tolist()
+        best = None
+        for _ in range(4):
+            runner.add_request("p")
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            runner.step([StepEntry("p", toks, [T - 1])], greedy=True)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t
+            runner.free_request("p")
+            best = dt if best is None else min(best, dt)
+        res["prefill_tok_s"] = round(T / best, 1)
+        res["prefill_ms"] = round(best * 1e3, 3)
+        del runner
+        for batch in sorted({1, args.batch}):
+            steps, warm, context = args.steps, args.warmup, args.context
+            runner = ModelRunner(model, page_size=P, num_pages=batch * ((context + P - 1) // P + 1), max_requests=batch)
+            start = context - (warm + steps)
+            for r in range(batch):
+                runner.add_request(r)
+                toks = torch.randint(0, V, (start,), generator=g).tolist()
+                for a in range(0, start, 2048):
+                    runner.step([StepEntry(r, toks[a:a + 2048], [])])
+            tokens = torch.randint(0, V, (batch,), generator=g).tolist()
+            for i in range(warm + steps):
+                if i == warm:
+                    torch.cuda.synchronize()
+                    t = time.perf_counter()
+                tokens = runner.step([StepEntry(r, [tokens[r]], [0]) for r in range(batch)], greedy=True)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t
+            res[f"decode_b{batch}_tok_s"] = round(batch * steps / dt, 1)
+            res[f"decode_b{batch}_ms_per_step"] = round(dt / steps * 1e3, 4)
+            res[f"decode_b{batch}_graph_steps"] = runner.graph_steps
+            del runner
+            torch.cuda.empty_cache()
+        del model
+        torch.cuda.empty_cache()
+        return res
+
+    out = {}
+    for name in [n for n in args.design_sizes.split(",") if n]:
+        z = ZARORAX_SIZES[name]
+        zcfg = config_from_dict(zarorax_config(z, layers, V))
+        qcfg = config_from_dict(dict(QWEN3_0_6B, vocab_size=V, hidden_size=z["width"], intermediate_size=z["top"] * z["expert_ff"],
+                                     num_hidden_layers=layers, num_attention_heads=z["heads"], num_key_value_heads=z["heads"] // 4,
+                                     head_dim=128, tie_word_embeddings=False))
+        out[name] = {"sizes": dict(z, layers=layers, vocab=V), "zarorax": measure(zcfg), "qwen3": measure(qcfg)}
+        print(f"[bench] {name}: {out[name]}", file=sys.stderr, flush=True)
+    first = next(iter(out.values()))
+    line = {"metric": f"decode tok/s @ batch {args.batch} (Zarorax, context {args.context}) beside Qwen3 of equal sizes",
+            "value": first["zarorax"][f"decode_b{args.batch}_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": first["zarorax"][f"decode_b{args.batch}_ms_per_step"],
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
+            "data": "synthetic: random weights, uniform-random token ids",
+            "config": {"model": "Zarorax and Qwen3 layer sizes (random weights)", "global_batch": args.batch,
+                       "seq_len": args.context, "prefill_tokens": args.prefill_tokens, "page_size": P, "parallelism": "single GPU"},
+            "designs": out}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def main() -> int:
     args = parse()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only: --gpus {args.gpus} is not supported (the engine has no multi-GPU path)")
         return 2
+    if args.design:
+        import qwen_engine_amd  # noqa: F401
+        return design_compare(args)
     import torch
     import qwen_engine_amd  # noqa: F401
     from qwen_engine_amd.config import Qwen3Config
