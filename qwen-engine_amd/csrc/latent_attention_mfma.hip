@@ -1,0 +1,286 @@
+// Attention over one cached latent per token on the matrix units (bfloat16), for prompts' portions and
+// for single new tokens alike.  See latent_attention.hip for the contract: packed queries
+// qp [T, H, R + Dr], cache rows [R + Dr] of which the first R are also the value, out [T, H, R].
+//
+// All heads read the same rows, so a wave's 16 columns are 16 heads of one token, and a block's four waves
+// are head groups of one token (few rows in the step, or many heads) or consecutive tokens (many rows).
+// The block walks the keys 32 at a time.  All its threads bring a tile from the cache into shared memory
+// twice: row-major, K[key][d], the A operand of S^T = K Q^T (v_mfma_f32_16x16x32_bf16, contraction over d),
+// and transposed, V^T[d][key], the A operand of O^T += V^T P^T (contraction over the 32 keys).  The
+// transposed copy is what a row-major cache costs: a lane's operand wants eight keys of one d side by side.
+// A thread loads four rows' 16 bytes and writes them back as eight 8-byte columns.  The keys of a tile are
+// kept in the order in which the scores come out of the first product (lane row g holds keys 4 g .. 4 g + 3
+// and 16 + 4 g .. 16 + 4 g + 3), so the weights go into the second product from the registers they are in.
+//
+// Tokens of a block that belong to different requests (the border between two portions, or single
+// tokens of a batch when the step has many rows) are served one request after the other: the waves of the
+// others wait at the barriers.
+//
+// The keys are cut into NS splits (a grid dimension; the same number for every token of the step, so a
+// recorded step needs no knowledge of the positions): split s of a token group whose last position is p
+// takes the keys [s L, (s + 1) L), L = ceil((p + 1) / NS) rounded up to 32.  With NS > 1 the splits' partial
+// results (running maximum, sum, unnormalised output, 32-bit) go to a workspace and a second kernel merges
+// them in the order of s.
+#include "attention_tile.h"
+
+#define LAT_VT_PITCH 40      // bf16 per row of the transposed tile: 32 keys and 8 of padding
+
+template <int RB, int DKC>
+__global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
+    const bf16_t* __restrict__ qp, bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml,
+    const bf16_t* __restrict__ cache, const int* __restrict__ positions, const int* __restrict__ tok_seq,
+    const int* __restrict__ block_table, int max_blocks, int T, int H, int R, int Dk, int P, float scale,
+    int TOK, int HGB, int NS) {
+    extern __shared__ __attribute__((aligned(16))) char lds_raw[];
+    const int dkc = (Dk + 31) / 32, rb = (R + 15) / 16;
+    const int kpitch = dkc * 32 + 8;
+    bf16_t* Ck = (bf16_t*)lds_raw;                 // [32][kpitch]
+    bf16_t* VT = Ck + 32 * kpitch;                 // [rb * 16][LAT_VT_PITCH]
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
+    const int split = blockIdx.y;
+    const int HG = (H + 15) / 16;
+    const int wt = wave / HGB, whg = wave % HGB;
+    const int t0 = blockIdx.x * TOK;
+    const int t = t0 + wt;
+    const int hg = blockIdx.z * HGB + whg;
+    const bool unit_ok = wt < TOK && t < T && hg < HG;
+    const int head = hg * 16 + n;
+    const bool head_ok = unit_ok && head < H;
+
+    bf16x8 q[DKC];
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int c = 0; c < DKC; ++c) {
+        const int d = c * 32 + g * 8;
+        q[c] = (head_ok && d < Dk) ? *(const bf16x8*)(qp + ((long)t * H + head) * Dk + d) : zero8;
+    }
+    float m = -INFINITY, l = 0.f;
+    floatx4 acc[RB];
+#pragma unroll
+    for (int db = 0; db < RB; ++db) acc[db] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    int seg = 0;
+    while (seg < TOK && t0 + seg < T) {
+        const int req = tok_seq[t0 + seg];
+        int end = seg + 1;
+        while (end < TOK && t0 + end < T && tok_seq[t0 + end] == req) ++end;
+        const int kmax = positions[t0 + end - 1];                  // (positions rise within a request's rows)
+        const int L = ((kmax + NS) / NS + 31) & ~31;
+        const int k0 = split * L;
+        const int k1 = min(k0 + L, kmax + 1);
+        const bool mine = unit_ok && wt >= seg && wt < end;
+        const int p = mine ? positions[t] : -1;
+        const int* bt = block_table + (long)req * max_blocks;
+        for (int kk = k0; kk < k1; kk += 32) {
+            __syncthreads();
+            for (int it = tid; it < 8 * dkc * 4; it += 256) {
+                const int kg = it / (dkc * 4), d0 = (it % (dkc * 4)) * 8;
+                uint4 r[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int key = kk + kg * 4 + j;
+                    r[j] = make_uint4(0, 0, 0, 0);
+                    if (key < k1 && d0 < Dk) {
+                        const long row = (long)bt[key / P] * P + key % P;
+                        r[j] = *(const uint4*)(cache + row * Dk + d0);
+                    }
+                    *(uint4*)(Ck + (kg * 4 + j) * kpitch + d0) = r[j];
+                }
+                if (d0 < rb * 16) {
+                    const int i0 = (kg & 3) * 8 + (kg >= 4 ? 4 : 0);
+                    const bool value = d0 < R;
+                    const unsigned w[4][4] = {{r[0].x, r[0].y, r[0].z, r[0].w}, {r[1].x, r[1].y, r[1].z, r[1].w},
+                                              {r[2].x, r[2].y, r[2].z, r[2].w}, {r[3].x, r[3].y, r[3].z, r[3].w}};
+#pragma unroll
+                    for (int e2 = 0; e2 < 4; ++e2) {               // the words hold d0 + 2 e2 (low half) and d0 + 2 e2 + 1 (high)
+                        uint2 lo, hi;
+                        lo.x = (w[0][e2] & 0xffffu) | (w[1][e2] << 16);
+                        lo.y = (w[2][e2] & 0xffffu) | (w[3][e2] << 16);
+                        hi.x = (w[0][e2] >> 16) | (w[1][e2] & 0xffff0000u);
+                        hi.y = (w[2][e2] >> 16) | (w[3][e2] & 0xffff0000u);
+                        if (!value) lo = hi = make_uint2(0, 0);
+                        *(uint2*)(VT + (d0 + 2 * e2) * LAT_VT_PITCH + i0) = lo;
+                        *(uint2*)(VT + (d0 + 2 * e2 + 1) * LAT_VT_PITCH + i0) = hi;
+                    }
+                }
+            }
+            __syncthreads();
+            if (!mine) continue;
+            floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < DKC; ++c) {
+                if (c < dkc) {
+                    const bf16x8 a0 = *(const bf16x8*)(Ck + n * kpitch + c * 32 + g * 8);
+                    const bf16x8 a1 = *(const bf16x8*)(Ck + (16 + n) * kpitch + c * 32 + g * 8);
+                    s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, q[c], s0, 0, 0, 0);
+                    s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, q[c], s1, 0, 0, 0);
+                }
+            }
+            float sv[8];
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int ka = kk + g * 4 + j, kb = ka + 16;
+                sv[j] = (ka <= p && ka < k1) ? s0[j] * scale : -INFINITY;
+                sv[4 + j] = (kb <= p && kb < k1) ? s1[j] * scale : -INFINITY;
+                tmax = fmaxf(tmax, fmaxf(sv[j], sv[4 + j]));
+            }
+            tmax = max_over_lane_rows(tmax);
+            const float mn = fmaxf(m, tmax);
+            const float ref = (mn == -INFINITY) ? 0.f : mn;
+            const float alpha = __expf(m - ref);
+            bf16x8 pb;
+            float psum = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float pj = __expf(sv[e] - ref);
+                psum += pj;
+                pb[e] = (__bf16)pj;
+            }
+            l = l * alpha + psum;
+            m = mn;
+#pragma unroll
+            for (int db = 0; db < RB; ++db) {
+                if (db < rb) {
+                    const bf16x8 a = *(const bf16x8*)(VT + (db * 16 + n) * LAT_VT_PITCH + g * 8);
+                    acc[db] *= alpha;
+                    acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[db], 0, 0, 0);
+                }
+            }
+        }
+        if (mine) {
+            float ls = l;
+            ls += __shfl_xor(ls, 16, 64);
+            ls += __shfl_xor(ls, 32, 64);
+            if (head_ok) {
+                if (NS == 1) {
+                    const float inv = 1.f / ls;
+                    bf16_t* o = out + ((long)t * H + head) * R;
+#pragma unroll
+                    for (int db = 0; db < RB; ++db) {
+                        const int d = db * 16 + g * 4;
+                        if (d < R) {                       // (R is a multiple of 8: four numbers lie inside or outside together)
+                            const float v[4] = {acc[db][0] * inv, acc[db][1] * inv, acc[db][2] * inv, acc[db][3] * inv};
+                            Vec4<bf16_t>::store(o + d, v);
+                        }
+                    }
+                } else {
+                    const int RP = rb * 16;
+                    float* pa = part_acc + (((long)t * H + head) * NS + split) * RP;
+#pragma unroll
+                    for (int db = 0; db < RB; ++db)
+                        if (db < rb) *(floatx4*)(pa + db * 16 + g * 4) = acc[db];
+                    if (g == 0) {
+                        float* pm = part_ml + (((long)t * H + head) * NS + split) * 2;
+                        pm[0] = m;
+                        pm[1] = ls;
+                    }
+                }
+            }
+        }
+        seg = end;
+    }
+}
+
+// One wave per (token, head): the splits' partial results, in the order of the splits.
+__global__ __launch_bounds__(64) void latent_attention_merge_kernel(const float* __restrict__ part_acc,
+                                                                    const float* __restrict__ part_ml,
+                                                                    bf16_t* __restrict__ out, int NS, int R, int RP) {
+    const long th = blockIdx.x;
+    const float* pm = part_ml + th * NS * 2;
+    float M = -INFINITY;
+    for (int s = 0; s < NS; ++s) M = fmaxf(M, pm[2 * s]);
+    float L = 0.f;
+    for (int s = 0; s < NS; ++s) L += (pm[2 * s] == -INFINITY ? 0.f : __expf(pm[2 * s] - M)) * pm[2 * s + 1];
+    const float inv = 1.f / L;
+    for (int d = threadIdx.x; d < R; d += 64) {
+        float a = 0.f;
+        for (int s = 0; s < NS; ++s) {
+            const float w = pm[2 * s] == -INFINITY ? 0.f : __expf(pm[2 * s] - M);
+            a = fmaf(w, part_acc[(th * NS + s) * RP + d], a);
+        }
+        Elem<bf16_t>::store(out + th * R + d, a * inv);
+    }
+}
+
+static bool latent_mfma_fits(int R, int Dk, int& rbc, int& dkc) {
+    if (R <= 0 || Dk < R || R % 8 || Dk % 8) return false;
+    const int rb = (R + 15) / 16, dk = (Dk + 31) / 32;
+    if (rb <= 4 && dk <= 4) { rbc = 4; dkc = 4; return true; }
+    if (rb <= 8 && dk <= 6) { rbc = 8; dkc = 6; return true; }
+    if (rb <= 16 && dk <= 10) { rbc = 16; dkc = 10; return true; }
+    if (rb <= 32 && dk <= 20) { rbc = 32; dkc = 20; return true; }
+    return false;
+}
+
+extern "C" int qe_latent_attention_mfma_supported(int R, int Dr) {
+    int a, b;
+    return latent_mfma_fits(R, R + Dr, a, b) ? 1 : 0;
+}
+
+// How the step's rows are laid over blocks and the keys over splits: from the shapes alone.
+static void latent_plan(int T, int H, int& TOK, int& HGB, int& NS) {
+    const int HG = (H + 15) / 16;
+    HGB = HG < 4 ? HG : 4;
+    TOK = T <= 64 ? 1 : (4 / HGB > 1 ? 4 / HGB : 1);
+    const long blocks = (long)qe_cdiv(T, TOK) * qe_cdiv(HG, HGB);
+    NS = 1;
+    if (blocks < 256) {
+        NS = qe_cdiv(512, blocks);
+        const int cap = T <= 64 ? 32 : 8;
+        if (NS > cap) NS = cap;
+    }
+}
+
+extern "C" long qe_latent_attention_mfma_workspace_bytes(int T, int H, int R) {
+    int TOK, HGB, NS;
+    latent_plan(T, H, TOK, HGB, NS);
+    if (NS == 1) return 0;
+    const long RP = (long)((R + 15) / 16) * 16;
+    return (long)T * H * NS * (RP + 2) * sizeof(float);
+}
+
+extern "C" int qe_latent_attention_mfma(const void* qp, void* out, const void* cache, const int* positions,
+                                        const int* tok_seq, const int* block_table, int max_blocks, int T, int H,
+                                        int R, int Dr, int P, float scale, void* workspace, long workspace_bytes,
+                                        hipStream_t stream) {
+    int rbc, dkcc;
+    const int Dk = R + Dr;
+    QE_REQUIRE(latent_mfma_fits(R, Dk, rbc, dkcc), "latent_attention (mfma): sizes R=%d Dr=%d not taken", R, Dr);
+    QE_REQUIRE(H > 0 && P > 0, "latent_attention (mfma): bad sizes");
+    if (T == 0) return 0;
+    int TOK, HGB, NS;
+    latent_plan(T, H, TOK, HGB, NS);
+    const int HG = (H + 15) / 16;
+    const long RP = (long)((R + 15) / 16) * 16;
+    QE_REQUIRE(workspace_bytes >= qe_latent_attention_mfma_workspace_bytes(T, H, R), "latent_attention (mfma): workspace too small");
+    QE_REQUIRE(NS <= 65535 && qe_cdiv(HG, HGB) <= 65535, "latent_attention (mfma): grid too large");
+    float* part_acc = (float*)workspace;
+    float* part_ml = part_acc ? part_acc + (long)T * H * NS * RP : nullptr;
+    const int dkc = (Dk + 31) / 32, rb = (R + 15) / 16;
+    const size_t shmem = ((size_t)32 * (dkc * 32 + 8) + (size_t)rb * 16 * LAT_VT_PITCH) * sizeof(bf16_t);
+    dim3 grid(qe_cdiv(T, TOK), NS, qe_cdiv(HG, HGB));
+#define QE_LA(RB_, DKC_)                                                                                              \
+    do {                                                                                                              \
+        static bool attr_set = false;                                                                                 \
+        if (!attr_set) {                                                                                              \
+            hipFuncSetAttribute((const void*)latent_attention_mfma_kernel<RB_, DKC_>,                                 \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                              \
+            attr_set = true;                                                                                          \
+        }                                                                                                             \
+        latent_attention_mfma_kernel<RB_, DKC_><<<grid, 256, shmem, stream>>>(                                        \
+            (const bf16_t*)qp, (bf16_t*)out, part_acc, part_ml, (const bf16_t*)cache, positions, tok_seq, block_table, \
+            max_blocks, T, H, R, Dk, P, scale, TOK, HGB, NS);                                                         \
+    } while (0)
+    if (rbc == 4) QE_LA(4, 4);
+    else if (rbc == 8) QE_LA(8, 6);
+    else if (rbc == 16) QE_LA(16, 10);
+    else QE_LA(32, 20);
+#undef QE_LA
+    QE_LAUNCH_CHECK();
+    if (NS > 1) {
+        latent_attention_merge_kernel<<<T * H, 64, 0, stream>>>(part_acc, part_ml, (bf16_t*)out, NS, R, (int)RP);
+        QE_LAUNCH_CHECK();
+    }
+    return 0;
+}

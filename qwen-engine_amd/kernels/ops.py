@@ -85,6 +85,8 @@ def load_library():
         "qe_latent_kv_store": [vp, vp, f32, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp],
         "qe_latent_q_rotate": [vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, i32, vp],
         "qe_latent_attention": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, vp],
+        "qe_latent_attention_mfma_supported": [i32, i32],
+        "qe_latent_attention_mfma": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, vp, i64, vp],
         "qe_gemm_heads": [vp, i64, i64, vp, vp, i64, i64, vp, i32, i32, i32, i32, i32, i32, vp],
         "qe_moe_route": [vp, vp, vp, i32, i32, i32, i32, i32, vp],
         "qe_moe_sort": [vp, i32, i32, i32, vp, vp, vp, i32, vp],
@@ -106,6 +108,8 @@ def load_library():
     lib.qe_attention_decode_workspace_bytes.argtypes = [i32, i32, i32, i32, i32]
     lib.qe_attention_decode_workspace_bytes.restype = ctypes.c_long
     lib.qe_attention_prefill_workspace_bytes.restype = ctypes.c_long
+    lib.qe_latent_attention_mfma_workspace_bytes.argtypes = [i32, i32, i32]
+    lib.qe_latent_attention_mfma_workspace_bytes.restype = ctypes.c_long
     lib.qe_attention_prefill_workspace_bytes_for.restype = ctypes.c_long
     _lib = lib
     return lib
@@ -923,9 +927,12 @@ def latent_q_rotate(q: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Te
 
 
 def latent_attention(qp: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok_seq: torch.Tensor,
-                     block_table: torch.Tensor, latent: int, scale: float) -> torch.Tensor:
+                     block_table: torch.Tensor, latent: int, scale: float, algo: int = ALGO_AUTO) -> torch.Tensor:
     """qp [T, H, R + Dr], cache [pages, 1, 1, P, R + Dr]: per (token, head) softmax(scale * qp . rows) . rows[:R]
-    over the rows at positions 0 .. p of request tok_seq[t] -> [T, H, R].  32-bit scores and weights."""
+    over the rows at positions 0 .. p of request tok_seq[t] -> [T, H, R].  32-bit scores and weights.  The rows
+    of a request are consecutive and their positions rise.  bfloat16 goes to the kernel on the matrix units
+    where it takes the sizes (multiples of 8, a latent of at most 512; the weights are rounded to bfloat16
+    before they meet the values), everything else (and ALGO_GENERIC) to the kernel on the vector units."""
     lib = load_library()
     _need(qp, "qp", _ACT, (None, None, None))
     T, H, D = qp.shape
@@ -937,6 +944,13 @@ def latent_attention(qp: torch.Tensor, cache: torch.Tensor, positions: torch.Ten
     _need(tok_seq, "tok_seq", torch.int32, (T,), dev)
     _need(block_table, "block_table", torch.int32, (None, None), dev)
     out = torch.empty((T, H, R), dtype=qp.dtype, device=dev)
+    if qp.dtype == torch.bfloat16 and algo != ALGO_GENERIC and lib.qe_latent_attention_mfma_supported(R, D - R):
+        nbytes = lib.qe_latent_attention_mfma_workspace_bytes(T, H, R)
+        ws = torch.empty((nbytes,), dtype=torch.uint8, device=dev) if nbytes else None
+        _check(lib.qe_latent_attention_mfma(qp.data_ptr(), out.data_ptr(), cache.data_ptr(), positions.data_ptr(),
+                                            tok_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, H, R,
+                                            D - R, P, float(scale), _ptr(ws), nbytes, _stream()), "latent_attention (mfma)")
+        return out
     _check(lib.qe_latent_attention(qp.data_ptr(), out.data_ptr(), cache.data_ptr(), positions.data_ptr(),
                                    tok_seq.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, H, R, D - R, P,
                                    float(scale), _DT[qp.dtype], _stream()), "latent_attention")

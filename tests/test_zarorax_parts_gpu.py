@@ -237,3 +237,38 @@ def test_experts_over_rows_grouped_on_the_device(dtype, tol, T):
     # a token's result does not depend on the batch around it
     alone = ops().moe_experts(x[:1].to(DEV), ids[:1].contiguous(), weights[:1].contiguous(), wgu, wd, limit, 1.702)
     assert torch.equal(alone[:, 0].cpu(), parts[:, 0].cpu())
+
+
+@pytest.mark.parametrize("R,Dr,H,P,lengths,new", [
+    (512, 64, 16, 16, [300, 1, 77], [300, 1, 77]),        # whole prompts side by side, many rows: tokens share a block
+    (512, 64, 16, 16, [700, 33, 64, 65, 129], [1, 1, 1, 1, 1]),   # single new tokens: the keys are cut into splits
+    (256, 32, 128, 8, [90, 200], [3, 70]),                # many heads: several head groups per token
+    (128, 32, 5, 16, [40, 41, 260], [40, 2, 100]),        # fewer heads than a wave has columns; mixed step
+    (64, 0, 24, 4, [130, 19], [130, 1]),                  # no rotated part; heads that fill one group and half of the next
+    (200, 24, 8, 32, [150], [150]),                       # sizes that are no multiple of 16 or 32
+])
+def test_latent_attention_on_the_matrix_units(R, Dr, H, P, lengths, new):
+    """The kernel on the matrix units against 64-bit torch, with the requests' last ``new`` tokens as the
+    step's rows: portions beside single tokens, borders between requests inside a block of rows."""
+    cache, table, rows = _latent_case(torch.bfloat16, R, Dr, H, P, lengths, seed=R + H + len(lengths))
+    g = torch.Generator().manual_seed(2)
+    qs, pos, seq = [], [], []
+    for b, (n, k) in enumerate(zip(lengths, new)):
+        for p in range(n - k, n):
+            qs.append(torch.randn(H, R + Dr, generator=g))
+            pos.append(p)
+            seq.append(b)
+    qp = torch.stack(qs).bfloat16()
+    scale = 1.5 / math.sqrt(R + Dr)
+    args = (qp.to(DEV), cache.to(DEV), torch.tensor(pos, dtype=torch.int32, device=DEV),
+            torch.tensor(seq, dtype=torch.int32, device=DEV), table.to(DEV), R, scale)
+    out = ops().latent_attention(*args)
+    plain = ops().latent_attention(*args, algo=ops().ALGO_GENERIC)
+    assert not torch.isnan(out.float()).any()
+    worst = 0.0
+    for i in range(0, len(pos), max(1, len(pos) // 40)):       # a sample of the rows against 64-bit arithmetic
+        keys = rows[seq[i]][:pos[i] + 1].double()
+        w = torch.softmax(qp[i].double() @ keys.t() * scale, dim=-1)
+        worst = max(worst, rel(out[i], w @ keys[:, :R]))
+    assert worst < 1.5e-2, worst
+    assert rel(out, plain.double().cpu()) < 2e-2               # every row against the kernel on the vector units
