@@ -50,6 +50,15 @@ struct QkvTail {
     float eps;
     int Hq, Hkv, P;
     int lp;   // log2 P: the page size is a power of two, and a division by a number known only at run time costs dozens of instructions an item
+    // Rows grouped by expert (a mixture of experts): the block's row tile is entry blockIdx of ``tiles``
+    // (expert, first row, rows <= BM), of which the device knows how many there are (n_tiles); W holds
+    // one [N, K] matrix per expert.  A block beyond the tiles leaves at once, so the grid follows the
+    // shapes alone.  null: one matrix, M rows.
+    const int* tiles;
+    const int* n_tiles;
+    // With SILU: act_limit > 0 makes the activation min(g, limit) sigmoid(act_slope g) (clamp(u, -limit, limit) + 1)
+    // instead of silu(g) u.
+    float act_limit, act_slope;
 };
 
 // BIG (256 x 256 by four waves, one wave a SIMD, a wave's part 128 x 128): the accumulators fill the
@@ -91,6 +100,15 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
     } else {
         tile_m = blockIdx.x % tiles_m;
         tile_n = blockIdx.x / tiles_m;
+    }
+    if (tail.tiles) {
+        if (tile_m >= tail.n_tiles[0]) return;
+        const int expert = tail.tiles[3 * tile_m], first = tail.tiles[3 * tile_m + 1];
+        M = tail.tiles[3 * tile_m + 2];
+        x += (long)first * K;
+        w += (long)expert * N * K;
+        out += (long)first * (SILU ? N / 2 : N);
+        tile_m = 0;
     }
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
@@ -495,8 +513,14 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     if (SILU) {
-                        const float gt = acc[i][j][4 * bq + r], up = acc[i][j + (SILU ? 1 : 0)][4 * bq + r];
-                        v[r] = gt * __builtin_amdgcn_rcpf(1.f + __expf(-gt)) * up;   // rcp: within 1 ulp
+                        float gt = acc[i][j][4 * bq + r], up = acc[i][j + (SILU ? 1 : 0)][4 * bq + r];
+                        float slope = 1.f;
+                        if (tail.act_limit > 0.f) {
+                            gt = fminf(gt, tail.act_limit);
+                            up = fminf(fmaxf(up, -tail.act_limit), tail.act_limit) + 1.f;
+                            slope = tail.act_slope;
+                        }
+                        v[r] = gt * __builtin_amdgcn_rcpf(1.f + __expf(-slope * gt)) * up;   // rcp: within 1 ulp
                     } else {
                         v[r] = acc[i][j][4 * bq + r];
                     }
@@ -568,6 +592,49 @@ static int launch_mfma(const void* x, const void* w, const float* bias, void* ou
     QE_LAUNCH_CHECK();
     return 0;
 }
+
+// Rows grouped by expert against one matrix per expert (see QkvTail): tiles of 128 x 128.
+template <typename TO, bool SILU>
+static int launch_grouped(const void* x, const void* w, void* out, const int* tiles, const int* n_tiles,
+                          int max_tiles, int N, int K, float limit, float slope, hipStream_t stream) {
+    constexpr int BM = 128, BN = 128, BK = 64, NW = 4;
+    const int tiles_n = qe_cdiv(N, BN);
+    const long blocks = (long)max_tiles * tiles_n;
+    QE_REQUIRE(blocks > 0 && blocks <= 2147483647L, "mfma gemm (grouped): too many tiles");
+    const size_t shmem = 2 * (BM + BN) * (BK * 2 + 16);
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute((const void*)gemm_mfma_kernel<TO, BM, BN, BK, NW, 2, SILU, false>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        attr_set = true;
+    }
+    QkvTail tail{};
+    tail.tiles = tiles;
+    tail.n_tiles = n_tiles;
+    tail.act_limit = limit;
+    tail.act_slope = slope;
+    gemm_mfma_kernel<TO, BM, BN, BK, NW, 2, SILU, false><<<dim3((unsigned)blocks, 1), 64 * NW, shmem, stream>>>(
+        (const bf16_t*)x, (const bf16_t*)w, nullptr, (TO*)out, 0, N, K, max_tiles, tiles_n, K, 0, 0, 0, tail);
+    QE_LAUNCH_CHECK();
+    return 0;
+}
+
+// x [rows, K] in the order of the tiles (an expert's rows side by side), w [E, N, K], out [rows, N] (silu: w's
+// gate and up rows interleaved in blocks of 32, out [rows, N / 2], with the clamped activation when limit > 0).
+extern "C" int qe_gemm_mfma_grouped(const void* x, const void* w, void* out, const int* tiles, const int* n_tiles,
+                                    int max_tiles, int N, int K, int silu, float limit, float slope, int dt_o,
+                                    hipStream_t stream) {
+    QE_REQUIRE(K % 8 == 0 && K >= 64, "mfma gemm (grouped): K=%d", K);
+    QE_REQUIRE(!silu || N % 64 == 0, "mfma gemm (grouped): gate|up rows in blocks of 32");
+    if (max_tiles == 0) return 0;
+    if (silu) {
+        QE_REQUIRE(dt_o == QE_BF16, "mfma gemm (grouped): the activation is stored in bfloat16");
+        return launch_grouped<bf16_t, true>(x, w, out, tiles, n_tiles, max_tiles, N, K, limit, slope, stream);
+    }
+    if (dt_o == QE_F32) return launch_grouped<float, false>(x, w, out, tiles, n_tiles, max_tiles, N, K, 0.f, 1.f, stream);
+    return launch_grouped<bf16_t, false>(x, w, out, tiles, n_tiles, max_tiles, N, K, 0.f, 1.f, stream);
+}
+extern "C" int qe_gemm_mfma_grouped_tile_rows() { return 128; }
 
 static int choose_tile(int M, int N, int splits, bool with_256x256 = true) {
     // The shape is chosen by what the busiest compute unit gets: its number of tiles (they are dealt

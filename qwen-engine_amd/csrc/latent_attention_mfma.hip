@@ -182,23 +182,27 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     }
 }
 
-// One wave per (token, head): the splits' partial results, in the order of the splits.
+// One wave per (token, head): the splits' partial results, in the order of the splits.  Lane s fetches split
+// s's maximum and sum, so that the weights are there after one trip to memory.
 __global__ __launch_bounds__(64) void latent_attention_merge_kernel(const float* __restrict__ part_acc,
                                                                     const float* __restrict__ part_ml,
                                                                     bf16_t* __restrict__ out, int NS, int R, int RP) {
+    __shared__ float wgt[64];
     const long th = blockIdx.x;
+    const int lane = threadIdx.x;
     const float* pm = part_ml + th * NS * 2;
-    float M = -INFINITY;
-    for (int s = 0; s < NS; ++s) M = fmaxf(M, pm[2 * s]);
+    const float ms = lane < NS ? pm[2 * lane] : -INFINITY;
+    const float ls = lane < NS ? pm[2 * lane + 1] : 0.f;
+    const float M = wave_max(ms);
+    const float w = ms == -INFINITY ? 0.f : __expf(ms - M);
+    wgt[lane] = w;
+    __syncthreads();
     float L = 0.f;
-    for (int s = 0; s < NS; ++s) L += (pm[2 * s] == -INFINITY ? 0.f : __expf(pm[2 * s] - M)) * pm[2 * s + 1];
+    for (int s = 0; s < NS; ++s) L = fmaf(wgt[s], __shfl(ls, s, 64), L);      // in the order of the splits
     const float inv = 1.f / L;
-    for (int d = threadIdx.x; d < R; d += 64) {
+    for (int d = lane; d < R; d += 64) {
         float a = 0.f;
-        for (int s = 0; s < NS; ++s) {
-            const float w = pm[2 * s] == -INFINITY ? 0.f : __expf(pm[2 * s] - M);
-            a = fmaf(w, part_acc[(th * NS + s) * RP + d], a);
-        }
+        for (int s = 0; s < NS; ++s) a = fmaf(wgt[s], part_acc[(th * NS + s) * RP + d], a);
         Elem<bf16_t>::store(out + th * R + d, a * inv);
     }
 }
@@ -254,7 +258,7 @@ extern "C" int qe_latent_attention_mfma(const void* qp, void* out, const void* c
     const int HG = (H + 15) / 16;
     const long RP = (long)((R + 15) / 16) * 16;
     QE_REQUIRE(workspace_bytes >= qe_latent_attention_mfma_workspace_bytes(T, H, R), "latent_attention (mfma): workspace too small");
-    QE_REQUIRE(NS <= 65535 && qe_cdiv(HG, HGB) <= 65535, "latent_attention (mfma): grid too large");
+    QE_REQUIRE(NS <= 64 && qe_cdiv(HG, HGB) <= 65535, "latent_attention (mfma): grid too large");
     float* part_acc = (float*)workspace;
     float* part_ml = part_acc ? part_acc + (long)T * H * NS * RP : nullptr;
     const int dkc = (Dk + 31) / 32, rb = (R + 15) / 16;

@@ -8,6 +8,9 @@
 //                  they are.  On ties the lower index wins.  ids [T, top], weights [T, top].
 //   qe_moe_sort    perm [T * top]: the pairs (as index t * top + j) ordered by expert; tiles
 //                  [max_tiles, 3] = (expert, first sorted row, rows <= tile_rows) and their number.
+//   qe_moe_gather  xs[i] = x[perm[i] / top]: the pairs' rows side by side, for a product that wants its rows
+//                  contiguous; qe_moe_combine  out[t] = sum_j weights[t, j] y[inv[t top + j]] in the order of j
+//                  (32-bit): the way back.
 //   qe_moe_gemm    for every tile, rows . W_e^T:
 //                    first product  (dual): x row of the pair's token against gate and up rows of
 //                      W_e [2 F, K]; g = min(g, limit), u = clamp(u, -limit, limit),
@@ -99,8 +102,8 @@ extern "C" int qe_moe_route(const float* logits, int* ids, float* weights, int T
 
 // One block.  n = T * top pairs.
 __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ ids, int n, int E, int tile_rows,
-                                                        int* __restrict__ perm, int* __restrict__ tiles,
-                                                        int* __restrict__ n_tiles) {
+                                                        int* __restrict__ perm, int* __restrict__ inv,
+                                                        int* __restrict__ tiles, int* __restrict__ n_tiles) {
     extern __shared__ int sm[];
     int* counts = sm;
     int* start = sm + E;
@@ -128,15 +131,20 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ 
         if (e == E - 1) n_tiles[0] = tb + mine;
     }
     __syncthreads();
-    for (int i = tid; i < n; i += blockDim.x) perm[atomicAdd(&cursor[ids[i]], 1)] = i;
+    for (int i = tid; i < n; i += blockDim.x) {
+        const int at = atomicAdd(&cursor[ids[i]], 1);
+        perm[at] = i;
+        if (inv) inv[i] = at;
+    }
 }
 
-extern "C" int qe_moe_sort(const int* ids, int n, int E, int tile_rows, int* perm, int* tiles, int* n_tiles,
+// inv (may be null): the sorted row of every pair, perm's inverse
+extern "C" int qe_moe_sort(const int* ids, int n, int E, int tile_rows, int* perm, int* inv, int* tiles, int* n_tiles,
                            int max_tiles, hipStream_t stream) {
     QE_REQUIRE(n >= 0 && E > 0 && tile_rows > 0, "moe_sort: bad sizes");
     QE_REQUIRE(max_tiles >= (n + tile_rows - 1) / tile_rows + (E < n ? E : n), "moe_sort: %d tiles may not be enough", max_tiles);
     QE_REQUIRE(3 * E * sizeof(int) <= 60000, "moe_sort: too many experts");
-    moe_sort_kernel<<<1, 1024, 3 * E * sizeof(int), stream>>>(ids, n, E, tile_rows, perm, tiles, n_tiles);
+    moe_sort_kernel<<<1, 1024, 3 * E * sizeof(int), stream>>>(ids, n, E, tile_rows, perm, inv, tiles, n_tiles);
     QE_LAUNCH_CHECK();
     return 0;
 }
@@ -148,7 +156,7 @@ template <typename TA, typename TW, bool DUAL>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(
     const TA* __restrict__ x, const int* __restrict__ perm, int top, const TW* __restrict__ w, void* __restrict__ out_,
     const float* __restrict__ weights, const int* __restrict__ tiles, const int* __restrict__ n_tiles, int T, int N,
-    int K, float limit, float slope) {
+    int K, float limit, float slope, int interleaved) {
     if ((int)blockIdx.y >= n_tiles[0]) return;
     __shared__ float xs[MK][MT + 4];
     __shared__ float ws[MK][MT + 4];
@@ -178,8 +186,11 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
             const int k = k0 + lk + i;
             const int n = n0 + lr;
             xs[lk + i][lr] = (xrow >= 0 && k < K) ? Elem<TA>::load(x + (long)xrow * K + k) : 0.f;
-            ws[lk + i][lr] = (n < N && k < K) ? Elem<TW>::load(we + (long)n * K + k) : 0.f;
-            if (DUAL) wu[lk + i][lr] = (n < N && k < K) ? Elem<TW>::load(we + (long)(N + n) * K + k) : 0.f;
+            // (gate and up rows one after the other, or in alternating blocks of 32)
+            const long ng = (DUAL && interleaved) ? (long)(n / 32) * 64 + n % 32 : n;
+            const long nu = (DUAL && interleaved) ? ng + 32 : (long)N + n;
+            ws[lk + i][lr] = (n < N && k < K) ? Elem<TW>::load(we + ng * K + k) : 0.f;
+            if (DUAL) wu[lk + i][lr] = (n < N && k < K) ? Elem<TW>::load(we + nu * K + k) : 0.f;
         }
         __syncthreads();
 #pragma unroll
@@ -229,18 +240,19 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
     }
 }
 
-// dual != 0: x [T, K] rows of the pairs' tokens, w [E, 2 N, K], out [T * top, N] in x's type at the sorted rows.
+// dual != 0: x [T, K] rows of the pairs' tokens, w [E, 2 N, K] (gate rows then up rows, or, interleaved, in
+// alternating blocks of 32), out [T * top, N] in x's type at the sorted rows.
 // dual == 0: x [T * top, K] sorted rows, w [E, N, K], out float [top, T, N].
 extern "C" int qe_moe_gemm(const void* x, const int* perm, int top, const void* w, void* out, const float* weights,
                            const int* tiles, const int* n_tiles, int max_tiles, int T, int N, int K, float limit,
-                           float slope, int dual, int dt_a, int dt_w, hipStream_t stream) {
+                           float slope, int dual, int interleaved, int dt_a, int dt_w, hipStream_t stream) {
     QE_REQUIRE(T >= 0 && N > 0 && K > 0 && top > 0 && max_tiles >= 0 && max_tiles <= 65535, "moe_gemm: bad sizes");
     if (T == 0 || max_tiles == 0) return 0;
     dim3 grid(qe_cdiv(N, MT), max_tiles);
 #define QE_MG(TA_, TW_)                                                                                              \
     do {                                                                                                             \
-        if (dual) moe_gemm_kernel<TA_, TW_, true><<<grid, 256, 0, stream>>>((const TA_*)x, perm, top, (const TW_*)w, out, weights, tiles, n_tiles, T, N, K, limit, slope); \
-        else moe_gemm_kernel<TA_, TW_, false><<<grid, 256, 0, stream>>>((const TA_*)x, perm, top, (const TW_*)w, out, weights, tiles, n_tiles, T, N, K, limit, slope);     \
+        if (dual) moe_gemm_kernel<TA_, TW_, true><<<grid, 256, 0, stream>>>((const TA_*)x, perm, top, (const TW_*)w, out, weights, tiles, n_tiles, T, N, K, limit, slope, interleaved); \
+        else moe_gemm_kernel<TA_, TW_, false><<<grid, 256, 0, stream>>>((const TA_*)x, perm, top, (const TW_*)w, out, weights, tiles, n_tiles, T, N, K, limit, slope, interleaved);     \
     } while (0)
     if (dt_a == QE_F32 && dt_w == QE_F32) QE_MG(float, float);
     else if (dt_a == QE_BF16 && dt_w == QE_BF16) QE_MG(bf16_t, bf16_t);
@@ -251,3 +263,45 @@ extern "C" int qe_moe_gemm(const void* x, const int* perm, int top, const void* 
 }
 
 extern "C" int qe_moe_tile_rows() { return MT; }
+
+template <typename TA>
+__global__ void moe_gather_kernel(const TA* __restrict__ x, const int* __restrict__ perm, int top, TA* __restrict__ xs, int K) {
+    const long i = blockIdx.x;
+    const TA* src = x + (long)(perm[i] / top) * K;
+    TA* dst = xs + i * K;
+    if ((K * sizeof(TA)) % 16 == 0) {
+        const int n16 = K * sizeof(TA) / 16;
+        for (int c = threadIdx.x; c < n16; c += blockDim.x) ((uint4*)dst)[c] = ((const uint4*)src)[c];
+    } else {
+        for (int c = threadIdx.x; c < K; c += blockDim.x) dst[c] = src[c];
+    }
+}
+
+extern "C" int qe_moe_gather(const void* x, const int* perm, int top, void* xs, int n, int K, int dt_a, hipStream_t stream) {
+    QE_REQUIRE(n >= 0 && K > 0 && top > 0, "moe_gather: bad sizes");
+    if (n == 0) return 0;
+    if (dt_a == QE_BF16) moe_gather_kernel<bf16_t><<<n, 128, 0, stream>>>((const bf16_t*)x, perm, top, (bf16_t*)xs, K);
+    else if (dt_a == QE_F32) moe_gather_kernel<float><<<n, 128, 0, stream>>>((const float*)x, perm, top, (float*)xs, K);
+    else QE_REQUIRE(false, "moe_gather: unknown type %d", dt_a);
+    QE_LAUNCH_CHECK();
+    return 0;
+}
+
+__global__ void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ inv, const float* __restrict__ weights,
+                                   float* __restrict__ out, int top, int H) {
+    const long t = blockIdx.x;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float a = 0.f;
+        for (int j = 0; j < top; ++j) a = fmaf(weights[t * top + j], y[(long)inv[t * top + j] * H + c], a);
+        out[t * H + c] = a;
+    }
+}
+
+extern "C" int qe_moe_combine(const float* y, const int* inv, const float* weights, float* out, int T, int top, int H,
+                              hipStream_t stream) {
+    QE_REQUIRE(T >= 0 && top > 0 && H > 0, "moe_combine: bad sizes");
+    if (T == 0) return 0;
+    moe_combine_kernel<<<T, 256, 0, stream>>>(y, inv, weights, out, top, H);
+    QE_LAUNCH_CHECK();
+    return 0;
+}

@@ -89,9 +89,15 @@ def load_library():
         "qe_latent_attention_mfma": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, vp, i64, vp],
         "qe_gemm_heads": [vp, i64, i64, vp, vp, i64, i64, vp, i32, i32, i32, i32, i32, i32, vp],
         "qe_moe_route": [vp, vp, vp, i32, i32, i32, i32, i32, vp],
-        "qe_moe_sort": [vp, i32, i32, i32, vp, vp, vp, i32, vp],
-        "qe_moe_gemm": [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, f32, i32, i32, i32, vp],
+        "qe_moe_sort": [vp, i32, i32, i32, vp, vp, vp, vp, i32, vp],
+        "qe_moe_gemm": [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, f32, i32, i32, i32, i32, vp],
+        "qe_moe_gather": [vp, vp, i32, vp, i32, i32, i32, vp],
+        "qe_moe_combine": [vp, vp, vp, vp, i32, i32, i32, vp],
+        "qe_gemm_mfma_grouped": [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, f32, i32, vp],
+        "qe_gemm_mfma_grouped_tile_rows": [],
         "qe_moe_tile_rows": [],
+        "qe_moe_gemm_mfma_supported": [i32],
+        "qe_moe_gemm_mfma": [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, f32, f32, i32, i32, vp],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)
@@ -995,10 +1001,19 @@ def moe_route(logits: torch.Tensor, groups: int, keep: int, top: int):
 
 
 def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor,
-                w_down: torch.Tensor, limit: float, slope: float) -> torch.Tensor:
-    """The chosen experts' outputs, weighted: float32 [top, T, H], the parts of a token's sum in the order of
-    its choices.  x [T, K]; w_gate_up [E, 2 F, K] (gate rows, then up rows); w_down [E, H, F].  An expert:
-    g = min(gate x, limit), u = clamp(up x, -limit, limit), down (g sigmoid(slope g) (u + 1))."""
+                w_down: torch.Tensor, limit: float, slope: float, interleaved: bool = False,
+                algo: int = ALGO_AUTO) -> torch.Tensor:
+    """The chosen experts' outputs, weighted: float32 [S, T, H] whose sum over S, in order, is the mixture's
+    output (S = top: a token's choices in their order; or S = 1: already added up in that order).
+    x [T, K]; w_gate_up [E, 2 F, K] (gate rows, then up rows; or, ``interleaved``, in alternating blocks of
+    32 as interleave_gate_up lays them); w_down [E, H, F].  An expert: g = min(gate x, limit),
+    u = clamp(up x, -limit, limit), down (g sigmoid(slope g) (u + 1)).
+
+    The (token, choice) pairs are grouped by expert on the device.  bfloat16 with many pairs: their rows are
+    gathered side by side and both products run on the tiled kernel of the dense products, a tile of 128
+    rows per block, every block finding its expert in the list of tiles.  bfloat16 with few pairs: a kernel
+    that reads its rows in place, tiles of 16 or 64 rows.  Otherwise (and ALGO_GENERIC) the kernel on the
+    vector units."""
     lib = load_library()
     _need(x, "x", _ACT, (None, None))
     T, K = x.shape
@@ -1011,19 +1026,51 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gat
     Fd = F2 // 2
     _need(w_down, "w_down", x.dtype, (E, None, Fd), dev)
     Hout = w_down.shape[1]
+    if interleaved and Fd % 32:
+        raise KernelError("moe_experts: interleaved gate|up rows come in blocks of 32")
     n = T * top
-    tile_rows = lib.qe_moe_tile_rows()
+    mfma = (x.dtype == torch.bfloat16 and algo != ALGO_GENERIC and lib.qe_moe_gemm_mfma_supported(K)
+            and lib.qe_moe_gemm_mfma_supported(Fd))
+    tiled = mfma and interleaved and n >= 1024 and K >= 64 and Fd >= 64
+    if tiled:
+        tile_rows = lib.qe_gemm_mfma_grouped_tile_rows()
+    elif mfma:
+        tile_rows = 16 if n <= 512 else 64
+    else:
+        tile_rows = lib.qe_moe_tile_rows()
     max_tiles = (n + tile_rows - 1) // tile_rows + min(E, n)
-    meta = torch.empty(n + 3 * max_tiles + 1, dtype=torch.int32, device=dev)
-    perm, tiles, n_tiles = meta[:n], meta[n:n + 3 * max_tiles], meta[n + 3 * max_tiles:]
-    _check(lib.qe_moe_sort(ids.data_ptr(), n, E, tile_rows, perm.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr(),
-                           max_tiles, _stream()), "moe_sort")
+    meta = torch.empty(2 * n + 3 * max_tiles + 1, dtype=torch.int32, device=dev)
+    perm, inv, tiles, n_tiles = meta[:n], meta[n:2 * n], meta[2 * n:2 * n + 3 * max_tiles], meta[2 * n + 3 * max_tiles:]
+    _check(lib.qe_moe_sort(ids.data_ptr(), n, E, tile_rows, perm.data_ptr(), inv.data_ptr(), tiles.data_ptr(),
+                           n_tiles.data_ptr(), max_tiles, _stream()), "moe_sort")
     a = torch.empty((n, Fd), dtype=x.dtype, device=dev)
+    if tiled:
+        xs = torch.empty((n, K), dtype=x.dtype, device=dev)
+        _check(lib.qe_moe_gather(x.data_ptr(), perm.data_ptr(), top, xs.data_ptr(), n, K, _DT[x.dtype], _stream()), "moe_gather")
+        _check(lib.qe_gemm_mfma_grouped(xs.data_ptr(), w_gate_up.data_ptr(), a.data_ptr(), tiles.data_ptr(),
+                                        n_tiles.data_ptr(), max_tiles, 2 * Fd, K, 1, float(limit), float(slope), BF16,
+                                        _stream()), "grouped gemm (gate, up)")
+        y = torch.empty((n, Hout), dtype=torch.float32, device=dev)
+        _check(lib.qe_gemm_mfma_grouped(a.data_ptr(), w_down.data_ptr(), y.data_ptr(), tiles.data_ptr(),
+                                        n_tiles.data_ptr(), max_tiles, Hout, Fd, 0, 0.0, 1.0, F32, _stream()),
+               "grouped gemm (down)")
+        out = torch.empty((1, T, Hout), dtype=torch.float32, device=dev)
+        _check(lib.qe_moe_combine(y.data_ptr(), inv.data_ptr(), weights.data_ptr(), out.data_ptr(), T, top, Hout,
+                                  _stream()), "moe_combine")
+        return out
+    parts = torch.empty((top, T, Hout), dtype=torch.float32, device=dev)
+    if mfma:
+        _check(lib.qe_moe_gemm_mfma(x.data_ptr(), perm.data_ptr(), top, w_gate_up.data_ptr(), a.data_ptr(), None,
+                                    tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, tile_rows, T, Fd, K, float(limit),
+                                    float(slope), 1, int(interleaved), _stream()), "moe_gemm (gate, up; mfma)")
+        _check(lib.qe_moe_gemm_mfma(a.data_ptr(), perm.data_ptr(), top, w_down.data_ptr(), parts.data_ptr(),
+                                    weights.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, tile_rows, T,
+                                    Hout, Fd, 0.0, 0.0, 0, 0, _stream()), "moe_gemm (down; mfma)")
+        return parts
     _check(lib.qe_moe_gemm(x.data_ptr(), perm.data_ptr(), top, w_gate_up.data_ptr(), a.data_ptr(), None,
                            tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, T, Fd, K, float(limit), float(slope), 1,
-                           _DT[x.dtype], _DT[w_gate_up.dtype], _stream()), "moe_gemm (gate, up)")
-    parts = torch.empty((top, T, Hout), dtype=torch.float32, device=dev)
+                           int(interleaved), _DT[x.dtype], _DT[w_gate_up.dtype], _stream()), "moe_gemm (gate, up)")
     _check(lib.qe_moe_gemm(a.data_ptr(), perm.data_ptr(), top, w_down.data_ptr(), parts.data_ptr(), weights.data_ptr(),
-                           tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, T, Hout, Fd, 0.0, 0.0, 0,
+                           tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, T, Hout, Fd, 0.0, 0.0, 0, 0,
                            _DT[x.dtype], _DT[w_down.dtype], _stream()), "moe_gemm (down)")
     return parts

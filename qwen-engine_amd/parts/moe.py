@@ -46,7 +46,7 @@ class GroupedMoE:
     largest scores among them (``ops.moe_route``); then the chosen experts' two products over the
     (token, choice) pairs grouped by expert on the device (``ops.moe_experts``).  The output is float32
     [top, T, H]: a token's weighted expert outputs in the order of its choices, which the norm that
-    follows adds to the stream."""
+    follows adds to the stream (or, with many rows, float32 [1, T, H]: already added up in that order)."""
     graph_safe = True
 
     def __init__(self, spec, hidden_size: int):
@@ -54,6 +54,9 @@ class GroupedMoE:
         self.hidden = int(hidden_size)
         self.e, self.top, self.inter = int(spec.num_experts), int(spec.top), int(spec.intermediate_size)
         self.w_router = self.w_gate_up = self.w_down = None
+        # gate and up rows in alternating blocks of 32 (what the tiled product's epilogue wants side by side)
+        # where the experts' width allows; else gate rows, then up rows
+        self.interleaved = self.inter % 32 == 0
 
     @staticmethod
     def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
@@ -72,8 +75,8 @@ class GroupedMoE:
         self.w_gate_up = torch.empty((self.e, 2 * self.inter, self.hidden), dtype=dt, device=rt.device)
         self.w_down = torch.empty((self.e, self.hidden, self.inter), dtype=dt, device=rt.device)
         for e in range(self.e):           # an expert at a time: the host never holds more
-            self.w_gate_up[e, :self.inter].copy_(tensors[f"e{e}.gate"])
-            self.w_gate_up[e, self.inter:].copy_(tensors[f"e{e}.up"])
+            g, u = tensors[f"e{e}.gate"], tensors[f"e{e}.up"]
+            self.w_gate_up[e].copy_(ops.interleave_gate_up(g, u) if self.interleaved else torch.cat([g, u], dim=0))
             self.w_down[e].copy_(tensors[f"e{e}.down"])
 
     def active_weight_bytes(self, tokens: int) -> int:
@@ -85,7 +88,7 @@ class GroupedMoE:
         s = self.spec
         logits = ops.gemm(x, self.w_router, out_dtype=torch.float32)
         ids, weights = ops.moe_route(logits, s.num_groups, s.keep_groups, s.top)
-        return ops.moe_experts(x, ids, weights, self.w_gate_up, self.w_down, s.limit, s.slope)
+        return ops.moe_experts(x, ids, weights, self.w_gate_up, self.w_down, s.limit, s.slope, interleaved=self.interleaved)
 
 
 register_part("polynorm_mlp", PolyNormMLP)
