@@ -88,3 +88,81 @@ extern "C" int qe_gemm_heads(const void* x, long xs_t, long xs_h, const void* w,
     QE_LAUNCH_CHECK();
     return 0;
 }
+
+// ---- the same on the matrix units (bfloat16, K a multiple of 8) -----------------------------------------------
+// out^T[n][t] = sum_k W_h[n][k] x[t][h][k] by v_mfma_f32_16x16x32_bf16: the head's weight rows are the A operand,
+// the tokens' rows the B operand, both read straight from memory in 16-byte pieces.  A block's four waves take
+// 16 output features each for MT * 16 tokens; blockIdx.z is the head.
+typedef __attribute__((ext_vector_type(8))) __bf16 gh_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float gh_floatx4;
+
+template <int MT>
+__global__ __launch_bounds__(256) void gemm_heads_mfma_kernel(
+    const bf16_t* __restrict__ x, long xs_t, long xs_h, const bf16_t* __restrict__ w, bf16_t* __restrict__ out, long os_t,
+    long os_h, const bf16_t* __restrict__ gate, int T, int N, int K) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, nn = lane & 15;
+    const int h = blockIdx.z, H = gridDim.z;
+    const int n_base = blockIdx.x * 64 + wave * 16;
+    if (n_base >= N) return;
+    const int t_base = blockIdx.y * MT * 16;
+    const int n_row = n_base + nn < N ? n_base + nn : N - 1;
+    const bf16_t* wr = w + ((long)h * N + n_row) * K + g * 8;
+    const bf16_t* xr[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int t = t_base + i * 16 + nn;
+        xr[i] = x + (long)(t < T ? t : T - 1) * xs_t + h * xs_h + g * 8;
+    }
+    gh_floatx4 acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[i] = gh_floatx4{0.f, 0.f, 0.f, 0.f};
+    const gh_bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll 2
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        const bool kin = k0 + g * 8 < K;
+        const gh_bf16x8 a = kin ? *(const gh_bf16x8*)(wr + k0) : zero8;
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const gh_bf16x8 b = kin ? *(const gh_bf16x8*)(xr[i] + k0) : zero8;
+            acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i], 0, 0, 0);
+        }
+    }
+    const int n0 = n_base + g * 4;     // lane (g, nn) holds token t_base + i * 16 + nn at the features n0 .. n0 + 3
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int t = t_base + i * 16 + nn;
+        if (t >= T) continue;
+        bf16_t* o = out + (long)t * os_t + h * os_h + n0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (n0 + j >= N) break;
+            float v = acc[i][j];
+            if (gate) {
+                const float gv = Elem<bf16_t>::load(gate + ((long)t * H + h) * N + n0 + j);
+                v = v / (1.f + __expf(-gv));
+            }
+            Elem<bf16_t>::store(o + j, v);
+        }
+    }
+}
+
+extern "C" int qe_gemm_heads_mfma_supported(int K, long xs_t, long xs_h) { return K > 0 && K % 8 == 0 && xs_t % 8 == 0 && xs_h % 8 == 0; }
+
+extern "C" int qe_gemm_heads_mfma(const void* x, long xs_t, long xs_h, const void* w, void* out, long os_t, long os_h,
+                                  const void* gate, int T, int H, int N, int K, hipStream_t stream) {
+    QE_REQUIRE(T >= 0 && H > 0 && N > 0 && qe_gemm_heads_mfma_supported(K, xs_t, xs_h), "gemm_heads (mfma): sizes not taken");
+    QE_REQUIRE(H <= 65535, "gemm_heads (mfma): too many heads");
+    if (T == 0) return 0;
+    if (T <= 32) {
+        dim3 grid(qe_cdiv(N, 64), qe_cdiv(T, 16), H);
+        gemm_heads_mfma_kernel<1><<<grid, 256, 0, stream>>>((const bf16_t*)x, xs_t, xs_h, (const bf16_t*)w, (bf16_t*)out,
+                                                             os_t, os_h, (const bf16_t*)gate, T, N, K);
+    } else {
+        QE_REQUIRE(qe_cdiv(T, 64) <= 65535, "gemm_heads (mfma): too many rows");
+        dim3 grid(qe_cdiv(N, 64), qe_cdiv(T, 64), H);
+        gemm_heads_mfma_kernel<4><<<grid, 256, 0, stream>>>((const bf16_t*)x, xs_t, xs_h, (const bf16_t*)w, (bf16_t*)out,
+                                                             os_t, os_h, (const bf16_t*)gate, T, N, K);
+    }
+    QE_LAUNCH_CHECK();
+    return 0;
+}

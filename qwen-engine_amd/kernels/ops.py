@@ -88,6 +88,8 @@ def load_library():
         "qe_latent_attention_mfma_supported": [i32, i32],
         "qe_latent_attention_mfma": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, vp, i64, vp],
         "qe_gemm_heads": [vp, i64, i64, vp, vp, i64, i64, vp, i32, i32, i32, i32, i32, i32, vp],
+        "qe_gemm_heads_mfma_supported": [i32, i64, i64],
+        "qe_gemm_heads_mfma": [vp, i64, i64, vp, vp, i64, i64, vp, i32, i32, i32, i32, vp],
         "qe_moe_route": [vp, vp, vp, i32, i32, i32, i32, i32, vp],
         "qe_moe_sort": [vp, i32, i32, i32, vp, vp, vp, vp, i32, vp],
         "qe_moe_gemm": [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, f32, i32, i32, i32, i32, vp],
@@ -963,7 +965,8 @@ def latent_attention(qp: torch.Tensor, cache: torch.Tensor, positions: torch.Ten
     return out
 
 
-def gemm_heads(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+def gemm_heads(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None,
+               algo: int = ALGO_AUTO) -> torch.Tensor:
     """out[t, h, :N] = w[h] x[t, h, :K] for w [H, N, K]; x [T, H, >= K] and out [T, H, >= N] (the product reads
     the first K and writes the first N numbers of each head).  gate [T, H * N]: the result times
     sigmoid(gate)."""
@@ -979,6 +982,11 @@ def gemm_heads(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Option
         raise KernelError("gemm_heads: 32-bit activations need 32-bit weights")
     if gate is not None:
         _need(gate, "gate", x.dtype, (T, H * N), x.device)
+    if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and algo != ALGO_GENERIC and
+            lib.qe_gemm_heads_mfma_supported(K, H * x.shape[2], x.shape[2])):
+        _check(lib.qe_gemm_heads_mfma(x.data_ptr(), H * x.shape[2], x.shape[2], w.data_ptr(), out.data_ptr(),
+                                      H * out.shape[2], out.shape[2], _ptr(gate), T, H, N, K, _stream()), "gemm_heads (mfma)")
+        return out
     _check(lib.qe_gemm_heads(x.data_ptr(), H * x.shape[2], x.shape[2], w.data_ptr(), out.data_ptr(),
                              H * out.shape[2], out.shape[2], _ptr(gate), T, H, N, K, _DT[x.dtype], _DT[w.dtype],
                              _stream()), "gemm_heads")

@@ -94,10 +94,10 @@ def test_short_convolution_continues_across_cuts_and_between_requests(taps):
 
 # ---- the products per head --------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-6), (torch.bfloat16, 8e-3)])
-def test_products_per_head_read_and_write_parts_of_wider_heads(dtype, tol):
+@pytest.mark.parametrize("T,H,K,N", [(37, 3, 20, 45), (5, 2, 24, 70), (130, 3, 64, 33), (64, 1, 128, 64)])
+def test_products_per_head_read_and_write_parts_of_wider_heads(dtype, tol, T, H, K, N):
     g = torch.Generator().manual_seed(5)
-    T, H, K, N = 37, 3, 20, 45
-    x = torch.randn(T, H, K + 6, generator=g).to(dtype)
+    x = torch.randn(T, H, K + 8, generator=g).to(dtype)
     w = (torch.randn(H, N, K, generator=g) / math.sqrt(K)).to(dtype)
     out = torch.full((T, H, N + 4), 9.0).to(dtype).to(DEV)
     ops().gemm_heads(x.to(DEV), w.to(DEV), out)
