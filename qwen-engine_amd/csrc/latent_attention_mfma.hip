@@ -23,7 +23,11 @@
 // them in the order of s.
 #include "attention_tile.h"
 
-#define LAT_VT_PITCH 40      // bf16 per row of the transposed tile: 32 keys and 8 of padding
+// bf16 per row of the transposed tile: 32 keys and 4 of padding, 18 words.  A thread writes eight rows that
+// lie eight rows apart from its neighbour's; with 18 words a row those land 16 banks apart (with 20 words, 32:
+// every write of the tile then met one of two banks and took thirty times as long).  A row starts at a
+// multiple of 8 bytes, so a lane's operand of 16 bytes is read as two halves.
+#define LAT_VT_PITCH 36
 
 template <int RB, int DKC>
 __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
@@ -74,7 +78,9 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
         for (int kk = k0; kk < k1; kk += 32) {
             __syncthreads();
             for (int it = tid; it < 8 * dkc * 4; it += 256) {
-                const int kg = it / (dkc * 4), d0 = (it % (dkc * 4)) * 8;
+                // (eight neighbouring lanes take the eight groups of four keys at the same d: their transposed
+                // writes fill a row of 64 bytes side by side)
+                const int kg = it & 7, d0 = (it >> 3) * 8;
                 uint4 r[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -142,7 +148,11 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
 #pragma unroll
             for (int db = 0; db < RB; ++db) {
                 if (db < rb) {
-                    const bf16x8 a = *(const bf16x8*)(VT + (db * 16 + n) * LAT_VT_PITCH + g * 8);
+                    union { bf16x8 v; uint2 h[2]; } au;
+                    const bf16_t* ap = VT + (db * 16 + n) * LAT_VT_PITCH + g * 8;
+                    au.h[0] = *(const uint2*)ap;
+                    au.h[1] = *(const uint2*)(ap + 4);
+                    const bf16x8 a = au.v;
                     acc[db] *= alpha;
                     acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, acc[db], 0, 0, 0);
                 }
