@@ -28,6 +28,7 @@
 // every write of the tile then met one of two banks and took thirty times as long).  A row starts at a
 // multiple of 8 bytes, so a lane's operand of 16 bytes is read as two halves.
 #define LAT_VT_PITCH 36
+#define LAT_CHUNK 512         // keys whose places in the cache are looked up at a time
 
 template <int RB, int DKC>
 __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
@@ -40,6 +41,9 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     const int kpitch = dkc * 32 + 8;
     bf16_t* Ck = (bf16_t*)lds_raw;                 // [32][kpitch]
     bf16_t* VT = Ck + 32 * kpitch;                 // [rb * 16][LAT_VT_PITCH]
+    __shared__ int rowoff[LAT_CHUNK];
+    constexpr int ITEMS = (8 * DKC * 4 + 255) / 256;   // pieces of four rows by eight numbers that a thread brings per tile
+    const int nitems = 8 * dkc * 4;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, g = lane >> 4, n = lane & 15;
     const int split = blockIdx.y;
     const int HG = (H + 15) / 16;
@@ -75,28 +79,44 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
         const bool mine = unit_ok && wt >= seg && wt < end;
         const int p = mine ? positions[t] : -1;
         const int* bt = block_table + (long)req * max_blocks;
-        for (int kk = k0; kk < k1; kk += 32) {
+        // The rows' places in the cache for up to LAT_CHUNK keys at a time, so that no load of a tile waits for
+        // the block table; a tile's loads are issued before the tile before it is computed and go to shared
+        // memory after it.
+        for (int kc = k0; kc < k1; kc += LAT_CHUNK) {
             __syncthreads();
-            for (int it = tid; it < 8 * dkc * 4; it += 256) {
+            for (int i = tid; i < LAT_CHUNK; i += 256) {
+                const int key = kc + i;
+                rowoff[i] = key < k1 ? bt[key / P] * P + key % P : 0;
+            }
+            __syncthreads();
+            const int kend = min(kc + LAT_CHUNK, k1);
+            uint4 r[ITEMS][4];
+#define LAT_ISSUE(kk_)                                                                                   \
+            _Pragma("unroll") for (int u = 0; u < ITEMS; ++u) {                                          \
+                const int it = tid + 256 * u, kg = it & 7, d0 = (it >> 3) * 8;                           \
+                _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                          \
+                    const int key = (kk_) + kg * 4 + j;                                                  \
+                    r[u][j] = make_uint4(0, 0, 0, 0);                                                    \
+                    if (it < nitems && key < k1 && d0 < Dk)                                              \
+                        r[u][j] = *(const uint4*)(cache + (long)rowoff[key - kc] * Dk + d0);             \
+                }                                                                                        \
+            }
+            LAT_ISSUE(kc)
+        for (int kk = kc; kk < kend; kk += 32) {
+            __syncthreads();
+#pragma unroll
+            for (int u = 0; u < ITEMS; ++u) {
                 // (eight neighbouring lanes take the eight groups of four keys at the same d: their transposed
                 // writes fill a row of 64 bytes side by side)
-                const int kg = it & 7, d0 = (it >> 3) * 8;
-                uint4 r[4];
+                const int it = tid + 256 * u, kg = it & 7, d0 = (it >> 3) * 8;
+                if (it >= nitems) continue;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int key = kk + kg * 4 + j;
-                    r[j] = make_uint4(0, 0, 0, 0);
-                    if (key < k1 && d0 < Dk) {
-                        const long row = (long)bt[key / P] * P + key % P;
-                        r[j] = *(const uint4*)(cache + row * Dk + d0);
-                    }
-                    *(uint4*)(Ck + (kg * 4 + j) * kpitch + d0) = r[j];
-                }
+                for (int j = 0; j < 4; ++j) *(uint4*)(Ck + (kg * 4 + j) * kpitch + d0) = r[u][j];
                 if (d0 < rb * 16) {
                     const int i0 = (kg & 3) * 8 + (kg >= 4 ? 4 : 0);
                     const bool value = d0 < R;
-                    const unsigned w[4][4] = {{r[0].x, r[0].y, r[0].z, r[0].w}, {r[1].x, r[1].y, r[1].z, r[1].w},
-                                              {r[2].x, r[2].y, r[2].z, r[2].w}, {r[3].x, r[3].y, r[3].z, r[3].w}};
+                    const unsigned w[4][4] = {{r[u][0].x, r[u][0].y, r[u][0].z, r[u][0].w}, {r[u][1].x, r[u][1].y, r[u][1].z, r[u][1].w},
+                                              {r[u][2].x, r[u][2].y, r[u][2].z, r[u][2].w}, {r[u][3].x, r[u][3].y, r[u][3].z, r[u][3].w}};
 #pragma unroll
                     for (int e2 = 0; e2 < 4; ++e2) {               // the words hold d0 + 2 e2 (low half) and d0 + 2 e2 + 1 (high)
                         uint2 lo, hi;
@@ -111,6 +131,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
                 }
             }
             __syncthreads();
+            if (kk + 32 < kend) { LAT_ISSUE(kk + 32) }
             if (!mine) continue;
             floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -158,6 +179,8 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
                 }
             }
         }
+        }
+#undef LAT_ISSUE
         if (mine) {
             float ls = l;
             ls += __shfl_xor(ls, 16, 64);
@@ -211,8 +234,17 @@ __global__ __launch_bounds__(64) void latent_attention_merge_kernel(const float*
     for (int s = 0; s < NS; ++s) L = fmaf(wgt[s], __shfl(ls, s, 64), L);      // in the order of the splits
     const float inv = 1.f / L;
     for (int d = lane; d < R; d += 64) {
+        const float* pa = part_acc + th * NS * RP + d;
         float a = 0.f;
-        for (int s = 0; s < NS; ++s) a = fmaf(wgt[s], part_acc[(th * NS + s) * RP + d], a);
+        int s = 0;
+        for (; s + 8 <= NS; s += 8) {                  // eight splits' loads together, added in the order of s
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = pa[(long)(s + u) * RP];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) a = fmaf(wgt[s + u], v[u], a);
+        }
+        for (; s < NS; ++s) a = fmaf(wgt[s], pa[(long)s * RP], a);
         Elem<bf16_t>::store(out + th * R + d, a * inv);
     }
 }
@@ -240,8 +272,8 @@ static void latent_plan(int T, int H, int& TOK, int& HGB, int& NS) {
     const long blocks = (long)qe_cdiv(T, TOK) * qe_cdiv(HG, HGB);
     NS = 1;
     if (blocks < 256) {
-        NS = qe_cdiv(512, blocks);
-        const int cap = T <= 64 ? 32 : 8;
+        NS = qe_cdiv(T <= 64 ? 1024 : 512, blocks);
+        const int cap = T <= 64 ? 64 : 8;
         if (NS > cap) NS = cap;
     }
 }
@@ -276,11 +308,13 @@ extern "C" int qe_latent_attention_mfma(const void* qp, void* out, const void* c
     dim3 grid(qe_cdiv(T, TOK), NS, qe_cdiv(HG, HGB));
 #define QE_LA(RB_, DKC_)                                                                                              \
     do {                                                                                                              \
-        static bool attr_set = false;                                                                                 \
-        if (!attr_set) {                                                                                              \
-            hipFuncSetAttribute((const void*)latent_attention_mfma_kernel<RB_, DKC_>,                                 \
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                              \
-            attr_set = true;                                                                                          \
+        static size_t attr_bytes = 48 * 1024;          /* (what a kernel may take without asking) */                 \
+        if (shmem > attr_bytes) {                                                                                     \
+            hipError_t e_ = hipFuncSetAttribute((const void*)latent_attention_mfma_kernel<RB_, DKC_>,                 \
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);              \
+            QE_REQUIRE(e_ == hipSuccess, "latent_attention (mfma): %zu bytes of shared memory: %s", shmem,             \
+                       hipGetErrorString(e_));                                                                        \
+            attr_bytes = shmem;                                                                                       \
         }                                                                                                             \
         latent_attention_mfma_kernel<RB_, DKC_><<<grid, 256, shmem, stream>>>(                                        \
             (const bf16_t*)qp, (bf16_t*)out, part_acc, part_ml, (const bf16_t*)cache, positions, tok_seq, block_table, \
