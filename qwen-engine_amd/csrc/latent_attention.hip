@@ -31,18 +31,37 @@ __device__ __forceinline__ void turn_pair(float angle, float& u, float& v) {
     v = b;
 }
 
+// q (may be null) [T, H, Dn + Dr] -> qp [T, H, R + Dr]: in the same launch, the rotated parts of the token's
+// queries go to the packed queries (what qe_latent_q_rotate does), so that a step of few rows has a kernel less.
 template <typename TC>
 __global__ void latent_kv_store_kernel(const float* __restrict__ kv, const float* __restrict__ weight, float eps,
                                        const int* __restrict__ positions, const float* __restrict__ inv_freq,
                                        int rot_dims, const int* __restrict__ slots, TC* __restrict__ cache,
-                                       int R, int Dr) {
+                                       int R, int Dr, const TC* __restrict__ q, TC* __restrict__ qp, int H, int Dn) {
     __shared__ float red[16];
     const long t = blockIdx.x;
+    if (q) {
+        const float pq = (float)positions[t];
+        const int pairs = (Dr + 1) / 2;
+        for (int idx = threadIdx.x; idx < H * pairs; idx += blockDim.x) {
+            const int h = idx / pairs, i = idx % pairs;
+            const TC* src = q + (t * H + h) * (Dn + Dr) + Dn;
+            TC* dst = qp + (t * H + h) * (R + Dr) + R;
+            if (2 * i + 1 >= Dr) {
+                Elem<TC>::store(dst + 2 * i, Elem<TC>::load(src + 2 * i));
+                continue;
+            }
+            float u = Elem<TC>::load(src + 2 * i), v = Elem<TC>::load(src + 2 * i + 1);
+            if (2 * i + 1 < rot_dims) turn_pair(pq * inv_freq[i], u, v);
+            Elem<TC>::store(dst + 2 * i, u);
+            Elem<TC>::store(dst + 2 * i + 1, v);
+        }
+    }
     const float* row = kv + t * (R + Dr);
     float ss = 0.f;
     for (int i = threadIdx.x; i < R; i += blockDim.x) ss += row[i] * row[i];
     ss = block_sum(ss, red);
-    const int slot = slots[t];
+    const int slot = slots ? slots[t] : -1;
     if (slot < 0) return;
     const float f = rsqrtf(ss / (float)R + eps);
     TC* dst = cache + (long)slot * (R + Dr);
@@ -59,17 +78,18 @@ __global__ void latent_kv_store_kernel(const float* __restrict__ kv, const float
 
 extern "C" int qe_latent_kv_store(const float* kv, const float* weight, float eps, const int* positions,
                                   const float* inv_freq, int rot_dims, const int* slots, void* cache, int dt_c,
-                                  int T, int R, int Dr, hipStream_t stream) {
+                                  int T, int R, int Dr, const void* q, void* qp, int H, int Dn, hipStream_t stream) {
+    QE_REQUIRE(!q || (qp && H > 0 && Dn >= 0), "latent_kv_store: queries without a place for them");
     QE_REQUIRE(T >= 0 && R > 0 && Dr >= 0, "latent_kv_store: bad sizes T=%d R=%d Dr=%d", T, R, Dr);
     QE_REQUIRE(rot_dims >= 0 && rot_dims <= Dr && rot_dims % 2 == 0, "latent_kv_store: %d rotated of %d", rot_dims, Dr);
     if (T == 0) return 0;
     const int threads = R >= 512 ? 256 : 64;
     if (dt_c == QE_F32)
         latent_kv_store_kernel<float><<<T, threads, 0, stream>>>(kv, weight, eps, positions, inv_freq, rot_dims, slots,
-                                                                  (float*)cache, R, Dr);
+                                                                  (float*)cache, R, Dr, (const float*)q, (float*)qp, H, Dn);
     else if (dt_c == QE_BF16)
         latent_kv_store_kernel<bf16_t><<<T, threads, 0, stream>>>(kv, weight, eps, positions, inv_freq, rot_dims, slots,
-                                                                   (bf16_t*)cache, R, Dr);
+                                                                   (bf16_t*)cache, R, Dr, (const bf16_t*)q, (bf16_t*)qp, H, Dn);
     else
         QE_REQUIRE(false, "latent_kv_store: unknown cache type %d", dt_c);
     QE_LAUNCH_CHECK();

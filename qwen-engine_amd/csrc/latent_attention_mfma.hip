@@ -84,9 +84,9 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
         // memory after it.
         for (int kc = k0; kc < k1; kc += LAT_CHUNK) {
             __syncthreads();
-            for (int i = tid; i < LAT_CHUNK; i += 256) {
+            for (int i = tid; i < LAT_CHUNK && kc + i < k1; i += 256) {
                 const int key = kc + i;
-                rowoff[i] = key < k1 ? bt[key / P] * P + key % P : 0;
+                rowoff[i] = bt[key / P] * P + key % P;
             }
             __syncthreads();
             const int kend = min(kc + LAT_CHUNK, k1);
@@ -270,10 +270,14 @@ static void latent_plan(int T, int H, int& TOK, int& HGB, int& NS) {
     HGB = HG < 4 ? HG : 4;
     TOK = T <= 64 ? 1 : (4 / HGB > 1 ? 4 / HGB : 1);
     const long blocks = (long)qe_cdiv(T, TOK) * qe_cdiv(HG, HGB);
+    // Splits: enough blocks to fill the chip, but every split of every (token, head) leaves R + 2 numbers for the
+    // merge to read again, so few rows get many splits and many rows few.
     NS = 1;
     if (blocks < 256) {
-        NS = qe_cdiv(T <= 64 ? 1024 : 512, blocks);
-        const int cap = T <= 64 ? 64 : 8;
+        NS = qe_cdiv(256, blocks);
+        int cap = T <= 64 ? 128 / T : 8;
+        if (cap < 8) cap = 8;
+        if (cap > 32) cap = 32;
         if (NS > cap) NS = cap;
     }
 }

@@ -58,6 +58,30 @@ __global__ void short_conv_update_kernel(const float* __restrict__ x, float* __r
     }
 }
 
+// Every row the only row of its request (single new tokens): the convolution and the state's shift in one launch;
+// a thread reads its channel's state, forms the output and writes the state back moved up by one.
+template <typename TA>
+__global__ void short_conv_single_kernel(const float* __restrict__ x, const float* __restrict__ w, float* __restrict__ state,
+                                         const int* __restrict__ tok_seq, TA* __restrict__ out, int H, int taps) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    const long t = blockIdx.y;
+    if (c >= H) return;
+    const int n1 = taps - 1;
+    float* st = state + (long)tok_seq[t] * n1 * H + c;
+    const float* wc = w + (long)c * taps;
+    const float xt = x[t * H + c];
+    float acc = xt;
+    for (int j = 0; j < n1; ++j) {                    // oldest input first, as in short_conv_kernel
+        const float v = st[(long)j * H];
+        acc = fmaf(wc[j], v, acc);
+        if (j > 0) st[(long)(j - 1) * H] = v;
+    }
+    acc = fmaf(wc[n1], xt, acc);
+    st[(long)(n1 - 1) * H] = xt;
+    Elem<TA>::store(out + t * H + c, acc);
+}
+
+// update 2: the caller knows that every row is the only row of its request
 extern "C" int qe_short_conv(const float* x, const float* w, float* state, const int* tok_seq, void* out,
                              int dt_a, int T, int H, int taps, int update, hipStream_t stream) {
     QE_REQUIRE(T >= 0 && H > 0 && taps >= 1, "short_conv: bad sizes T=%d H=%d taps=%d", T, H, taps);
@@ -66,6 +90,13 @@ extern "C" int qe_short_conv(const float* x, const float* w, float* state, const
     if (T == 0) return 0;
     const int threads = H >= 256 ? 256 : 64;
     dim3 grid(qe_cdiv(H, threads), T);                // (blockIdx.y is the row)
+    if (update == 2 && taps > 1) {
+        if (dt_a == QE_F32) short_conv_single_kernel<float><<<grid, threads, 0, stream>>>(x, w, state, tok_seq, (float*)out, H, taps);
+        else if (dt_a == QE_BF16) short_conv_single_kernel<bf16_t><<<grid, threads, 0, stream>>>(x, w, state, tok_seq, (bf16_t*)out, H, taps);
+        else QE_REQUIRE(false, "short_conv: unknown output type %d", dt_a);
+        QE_LAUNCH_CHECK();
+        return 0;
+    }
     if (dt_a == QE_F32)
         short_conv_kernel<float><<<grid, threads, 0, stream>>>(x, w, state, tok_seq, (float*)out, T, H, taps);
     else if (dt_a == QE_BF16)

@@ -82,7 +82,7 @@ def load_library():
         "qe_postnorm": [vp, vp, i32, i32, f32, vp, f32, vp, i32, i32, i32, vp],
         "qe_polynorm": [vp, vp, f32, vp, i32, i32, i32, vp],
         "qe_short_conv": [vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp],
-        "qe_latent_kv_store": [vp, vp, f32, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp],
+        "qe_latent_kv_store": [vp, vp, f32, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp, vp, i32, i32, vp],
         "qe_latent_q_rotate": [vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, i32, vp],
         "qe_latent_attention": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, vp],
         "qe_latent_attention_mfma_supported": [i32, i32],
@@ -874,11 +874,13 @@ def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float, out_dtype: torch.d
 
 
 def short_conv(x: torch.Tensor, w: torch.Tensor, state: Optional[torch.Tensor], tok_seq: torch.Tensor,
-               out_dtype: torch.dtype, update: bool = True) -> torch.Tensor:
+               out_dtype: torch.dtype, update: bool = True, single_rows: bool = False) -> torch.Tensor:
     """out_t = x_t + sum_k w[:, taps - 1 - k] x_(t - k) along each request's tokens, x the 32-bit stream
     [T, H], w float32 [H, taps].  What lies before a request's rows in this step comes from state
     (float32 [slots, taps - 1, H], row tok_seq[t]: the request's last taps - 1 inputs), which then takes
-    the step's last inputs (``update``).  The rows of a request are consecutive."""
+    the step's last inputs (``update``).  The rows of a request are consecutive.  ``single_rows``: the caller
+    knows that no two rows belong to the same request (single new tokens, each with a state row of its own):
+    convolution and update are then one launch."""
     lib = load_library()
     _need(x, "x", torch.float32, (None, None))
     T, H = x.shape
@@ -891,16 +893,19 @@ def short_conv(x: torch.Tensor, w: torch.Tensor, state: Optional[torch.Tensor], 
         _need(state, "state", torch.float32, (None, taps - 1, H), x.device)
     out = torch.empty((T, H), dtype=out_dtype, device=x.device)
     _check(lib.qe_short_conv(x.data_ptr(), w.data_ptr(), _ptr(state), tok_seq.data_ptr(), out.data_ptr(),
-                             _DT[out_dtype], T, H, taps, int(update), _stream()), "short_conv")
+                             _DT[out_dtype], T, H, taps, 2 if (update and single_rows) else int(update), _stream()),
+           "short_conv")
     return out
 
 
 # ---- attention over one cached latent per token --------------------------------------------------------
 def latent_kv_store(kv: torch.Tensor, weight: torch.Tensor, eps: float, positions: torch.Tensor,
-                    inv_freq: torch.Tensor, slots: torch.Tensor, cache: torch.Tensor) -> None:
+                    inv_freq: torch.Tensor, slots: Optional[torch.Tensor], cache: torch.Tensor,
+                    q: Optional[torch.Tensor] = None, qp: Optional[torch.Tensor] = None, dim: int = 0) -> None:
     """kv float32 [T, R + Dr] (R = weight's length): the first R normed (weight * u / rms(u)), the last Dr
     turned in neighbouring pairs by positions * inv_freq (float32 [n], 2 n <= Dr; the rest passes), into
-    the row slots[t] of cache [pages, 1, 1, P, R + Dr] (negative slot: nowhere)."""
+    the row slots[t] of cache [pages, 1, 1, P, R + Dr] (negative slot, or no slots: nowhere).  With q
+    [T, H, dim + Dr] and qp [T, H, R + Dr] the same launch does what latent_q_rotate does."""
     lib = load_library()
     _need(kv, "kv", torch.float32, (None, None))
     T, D = kv.shape
@@ -909,11 +914,17 @@ def latent_kv_store(kv: torch.Tensor, weight: torch.Tensor, eps: float, position
     R = weight.shape[0]
     _need(cache, "cache", _ACT, (None, 1, 1, None, D), dev)
     _need(positions, "positions", torch.int32, (T,), dev)
-    _need(slots, "slots", torch.int32, (T,), dev)
+    if slots is not None:
+        _need(slots, "slots", torch.int32, (T,), dev)
     _need(inv_freq, "inv_freq", torch.float32, (None,), dev)
+    H = 0
+    if q is not None:
+        _need(q, "q", cache.dtype, (T, None, int(dim) + D - R), dev)
+        H = q.shape[1]
+        _need(qp, "qp", cache.dtype, (T, H, D), dev)
     _check(lib.qe_latent_kv_store(kv.data_ptr(), weight.data_ptr(), float(eps), positions.data_ptr(),
-                                  inv_freq.data_ptr(), 2 * inv_freq.shape[0], slots.data_ptr(), cache.data_ptr(),
-                                  _DT[cache.dtype], T, R, D - R, _stream()), "latent_kv_store")
+                                  inv_freq.data_ptr(), 2 * inv_freq.shape[0], _ptr(slots), cache.data_ptr(),
+                                  _DT[cache.dtype], T, R, D - R, _ptr(q), _ptr(qp), H, int(dim), _stream()), "latent_kv_store")
 
 
 def latent_q_rotate(q: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, qp: torch.Tensor,

@@ -37,7 +37,9 @@ class ShortConv:
 
     def forward(self, x: torch.Tensor, ctx, state: Optional[torch.Tensor]) -> torch.Tensor:
         """x: the 32-bit stream [T, H]; state [slots, taps - 1, H], read and brought up to date."""
-        return ops.short_conv(x, self.weight, state, ctx.tok_seq, ctx.rt.dtype)
+        # (a step in which every request brings one token: convolution and the state's shift in one launch)
+        single = all(s.q_len == 1 for s in ctx.seqs) and len(ctx.seqs) == x.shape[0]
+        return ops.short_conv(x, self.weight, state, ctx.tok_seq, ctx.rt.dtype, single_rows=single)
 
 
 register_part("short_conv", ShortConv)

@@ -105,13 +105,14 @@ class LatentAttention:
         else:
             q = ops.gemm(x, self.w_q)
         q = q.view(T, self.h, self.dn + self.dr)
-        # the token's cache row: normed latent | rotated shared key part
+        # the token's cache row (normed latent | rotated shared key part) and the rotated parts of the packed
+        # queries [Uk^T q | rotated q], in one launch
+        qp = torch.empty((T, self.h, self.r + self.dr), dtype=dt, device=x.device)
         if binding.write:
             kv = ops.gemm(x, self.w_dkv, out_dtype=torch.float32)
-            ops.latent_kv_store(kv, self.kv_norm, self.eps, ctx.positions, inv_freq, ctx.slots[g], cache)
-        # packed queries [Uk^T q | rotated q]
-        qp = torch.empty((T, self.h, self.r + self.dr), dtype=dt, device=x.device)
-        ops.latent_q_rotate(q, ctx.positions, inv_freq, qp, self.dn)
+            ops.latent_kv_store(kv, self.kv_norm, self.eps, ctx.positions, inv_freq, ctx.slots[g], cache, q, qp, self.dn)
+        else:
+            ops.latent_q_rotate(q, ctx.positions, inv_freq, qp, self.dn)
         if self.dn > 0:
             ops.gemm_heads(q, self.w_uk_t, qp)
         else:
