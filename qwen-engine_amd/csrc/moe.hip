@@ -106,8 +106,7 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ 
                                                         int* __restrict__ tiles, int* __restrict__ n_tiles) {
     extern __shared__ int sm[];
     int* counts = sm;
-    int* start = sm + E;
-    int* cursor = sm + 2 * E;
+    int* cursor = sm + E;
     const int tid = threadIdx.x;
     for (int e = tid; e < E; e += blockDim.x) counts[e] = 0;
     __syncthreads();
@@ -119,7 +118,6 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ 
             off += counts[j];
             tb += (counts[j] + tile_rows - 1) / tile_rows;
         }
-        start[e] = off;
         cursor[e] = off;
         const int c = counts[e];
         const int mine = (c + tile_rows - 1) / tile_rows;
@@ -143,8 +141,8 @@ extern "C" int qe_moe_sort(const int* ids, int n, int E, int tile_rows, int* per
                            int max_tiles, hipStream_t stream) {
     QE_REQUIRE(n >= 0 && E > 0 && tile_rows > 0, "moe_sort: bad sizes");
     QE_REQUIRE(max_tiles >= (n + tile_rows - 1) / tile_rows + (E < n ? E : n), "moe_sort: %d tiles may not be enough", max_tiles);
-    QE_REQUIRE(3 * E * sizeof(int) <= 60000, "moe_sort: too many experts");
-    moe_sort_kernel<<<1, 1024, 3 * E * sizeof(int), stream>>>(ids, n, E, tile_rows, perm, inv, tiles, n_tiles);
+    QE_REQUIRE(2 * E * sizeof(int) <= 60000, "moe_sort: too many experts");
+    moe_sort_kernel<<<1, 1024, 2 * E * sizeof(int), stream>>>(ids, n, E, tile_rows, perm, inv, tiles, n_tiles);
     QE_LAUNCH_CHECK();
     return 0;
 }

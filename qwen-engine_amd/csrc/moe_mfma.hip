@@ -10,7 +10,10 @@
 // K is a multiple of 8; other sizes are arbitrary.
 #include "attention_tile.h"
 
-template <int MT, bool DUAL>
+// KSPLIT (with MT == 1, few rows): the block's four waves take the same 16 features and a quarter of K each
+// (steps of 32 in turn), and wave 0 adds the four parts in the order of the waves: four times the blocks, for
+// a product that is bound by streaming the weights of the few experts that a handful of tokens choose.
+template <int MT, bool DUAL, bool KSPLIT = false>
 __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(
     const bf16_t* __restrict__ x, const int* __restrict__ perm, int top, const bf16_t* __restrict__ w,
     void* __restrict__ out_, const float* __restrict__ weights, const int* __restrict__ tiles,
@@ -18,7 +21,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(
     if ((int)blockIdx.y >= n_tiles[0]) return;
     const int e = tiles[3 * blockIdx.y], r0 = tiles[3 * blockIdx.y + 1], rows = tiles[3 * blockIdx.y + 2];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, nn = lane & 15;
-    const int n_base = blockIdx.x * 64 + wave * 16;
+    const int n_base = KSPLIT ? blockIdx.x * 16 : blockIdx.x * 64 + wave * 16;
     if (n_base >= N) return;
     const int n_row = n_base + nn < N ? n_base + nn : N - 1;
     // (gate and up rows one after the other, or in alternating blocks of 32)
@@ -38,7 +41,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(
     for (int i = 0; i < MT; ++i) ag[i] = au[i] = floatx4{0.f, 0.f, 0.f, 0.f};
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll 2
-    for (int k0 = 0; k0 < K; k0 += 32) {
+    for (int k0 = KSPLIT ? wave * 32 : 0; k0 < K; k0 += KSPLIT ? 128 : 32) {
         const bool kin = k0 + g * 8 < K;
         const bf16x8 a = kin ? *(const bf16x8*)(wg + k0) : zero8;
         bf16x8 b = zero8;
@@ -48,6 +51,20 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(
             const bf16x8 xb = kin ? *(const bf16x8*)(xr[i] + k0) : zero8;
             ag[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, xb, ag[i], 0, 0, 0);
             if (DUAL) au[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b, xb, au[i], 0, 0, 0);
+        }
+    }
+    if (KSPLIT) {
+        __shared__ floatx4 part[3][2][64];
+        if (wave > 0) {
+            part[wave - 1][0][lane] = ag[0];
+            if (DUAL) part[wave - 1][1][lane] = au[0];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int v = 0; v < 3; ++v) {
+            ag[0] += part[v][0][lane];
+            if (DUAL) au[0] += part[v][1][lane];
         }
     }
     // lane (g, nn) holds the row m = i * 16 + nn at the features n_base + g * 4 + j
@@ -86,10 +103,13 @@ extern "C" int qe_moe_gemm_mfma(const void* x, const int* perm, int top, const v
     QE_REQUIRE(qe_moe_gemm_mfma_supported(K), "moe_gemm (mfma): K=%d is no multiple of 8", K);
     QE_REQUIRE(tile_rows == 16 || tile_rows == 64, "moe_gemm (mfma): tiles of %d rows", tile_rows);
     if (T == 0 || max_tiles == 0) return 0;
-    dim3 grid(qe_cdiv(N, 64), max_tiles);
-#define QE_MM(MT_, DUAL_) moe_gemm_mfma_kernel<MT_, DUAL_><<<grid, 256, 0, stream>>>((const bf16_t*)x, perm, top, (const bf16_t*)w, out, weights, tiles, n_tiles, T, N, K, limit, slope, interleaved)
-    if (tile_rows == 16) { if (dual) QE_MM(1, true); else QE_MM(1, false); }
-    else { if (dual) QE_MM(4, true); else QE_MM(4, false); }
+    // few tiles of 16 rows (single new tokens): K is shared out over a block's waves
+    const bool ksplit = tile_rows == 16 && max_tiles <= 64 && K >= 256;
+    dim3 grid(qe_cdiv(N, ksplit ? 16 : 64), max_tiles);
+#define QE_MM(MT_, DUAL_, KS_) moe_gemm_mfma_kernel<MT_, DUAL_, KS_><<<grid, 256, 0, stream>>>((const bf16_t*)x, perm, top, (const bf16_t*)w, out, weights, tiles, n_tiles, T, N, K, limit, slope, interleaved)
+    if (ksplit) { if (dual) QE_MM(1, true, true); else QE_MM(1, false, true); }
+    else if (tile_rows == 16) { if (dual) QE_MM(1, true, false); else QE_MM(1, false, false); }
+    else { if (dual) QE_MM(4, true, false); else QE_MM(4, false, false); }
 #undef QE_MM
     QE_LAUNCH_CHECK();
     return 0;
