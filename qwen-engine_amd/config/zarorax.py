@@ -73,10 +73,6 @@ class ZaroraxConfig:
                 if not (isinstance(src, int) and 0 <= src < len(self.layers)) or src == i or \
                         self.layers[src].get("weights_of") is not None:
                     raise ConfigError(f"{where}weights_of names layer {src!r}, which has no weights of its own")
-                other = self.layers[src]
-                if (layer.get("type"), layer.get("mixer"), layer.get("mlp")) != \
-                        (other.get("type"), other.get("mixer"), other.get("mlp")):
-                    raise ConfigError(f"{where}weights_of: the entry differs from layer {src}'s")
             self._mixer(layer, where)
             self._ffn(layer, where)
 

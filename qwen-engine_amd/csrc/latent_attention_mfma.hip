@@ -48,7 +48,9 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     const int split = blockIdx.y;
     const int HG = (H + 15) / 16;
     const int wt = wave / HGB, whg = wave % HGB;
-    const int t0 = blockIdx.x * TOK;
+    // (the step's last rows see the most keys: their blocks start first, so that no compute unit is left with a
+    // long block at the end)
+    const int t0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * TOK;
     const int t = t0 + wt;
     const int hg = blockIdx.z * HGB + whg;
     const bool unit_ok = wt < TOK && t < T && hg < HG;
