@@ -21,7 +21,7 @@
 // sine and cosine are 32-bit.
 #include "common.h"
 
-#define LAT_MAX_R 1024
+#define LAT_MAX_R 2048
 
 __device__ __forceinline__ void turn_pair(float angle, float& u, float& v) {
     float s, c;

@@ -39,6 +39,54 @@ __global__ void postnorm_kernel(float* __restrict__ x, const TD* __restrict__ de
     }
 }
 
+// The same for rows of up to NV * 4 * blockDim.x numbers with H % 4 == 0: the row is read once, in 16-byte
+// pieces, and kept in registers (a step of few rows is a chain of short kernels, each bound by its trips to memory).
+template <typename TA, typename TD, int NV>
+__global__ __launch_bounds__(256) void postnorm_regs_kernel(float* __restrict__ x, const TD* __restrict__ delta, int n_delta,
+                                                            long delta_stride, float alpha, const float* __restrict__ gain,
+                                                            float eps, TA* __restrict__ act, int H) {
+    __shared__ float red[16];
+    const long r = blockIdx.x;
+    float* xr = x + r * H;
+    const TD* dr = delta ? delta + r * H : nullptr;
+    float z[NV][4];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = (threadIdx.x + i * blockDim.x) * 4;
+        if (c < H) {
+            Vec4<float>::load(xr + c, z[i]);
+            float d[4] = {0.f, 0.f, 0.f, 0.f};
+            if (dr) {
+                Vec4<TD>::load(dr + c, d);
+                for (int s = 1; s < n_delta; ++s) {
+                    float e[4];
+                    Vec4<TD>::load(dr + s * delta_stride + c, e);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) d[k] += e[k];
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                z[i][k] = fmaf(alpha, z[i][k], d[k]);
+                ss += z[i][k] * z[i][k];
+            }
+        }
+    }
+    ss = block_sum(ss, red);
+    const float f = rsqrtf(ss / (float)H + eps) * gain[0];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int c = (threadIdx.x + i * blockDim.x) * 4;
+        if (c < H) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) z[i][k] *= f;
+            Vec4<float>::store(xr + c, z[i]);
+            if (act) Vec4<TA>::store(act + r * H + c, z[i]);
+        }
+    }
+}
+
 // dt_d: element type of delta; dt_a: of the copy (act may be null: no copy)
 extern "C" int qe_postnorm(float* x, const void* delta, int n_delta, int dt_d, float alpha, const float* gain,
                            float eps, void* act, int dt_a, int T, int H, hipStream_t stream) {
@@ -47,7 +95,15 @@ extern "C" int qe_postnorm(float* x, const void* delta, int n_delta, int dt_d, f
     if (T == 0) return 0;
     const long stride = (long)T * H;
     const int threads = H >= 2048 ? 512 : (H >= 512 ? 256 : 64);
-#define QE_PN(TA_, TD_) postnorm_kernel<TA_, TD_><<<T, threads, 0, stream>>>(x, (const TD_*)delta, n_delta, stride, alpha, gain, eps, (TA_*)act, H)
+    const bool regs = H % 4 == 0 && H <= 8192;
+    const int rthreads = regs ? (((H / 4 + 63) / 64) * 64 > 256 ? 256 : ((H / 4 + 63) / 64) * 64) : 0;
+    const int nv = regs ? (H / 4 + rthreads - 1) / rthreads : 0;
+#define QE_PN(TA_, TD_)                                                                                                       \
+    do {                                                                                                                      \
+        if (regs && nv <= 2) postnorm_regs_kernel<TA_, TD_, 2><<<T, rthreads, 0, stream>>>(x, (const TD_*)delta, n_delta, stride, alpha, gain, eps, (TA_*)act, H); \
+        else if (regs) postnorm_regs_kernel<TA_, TD_, 8><<<T, rthreads, 0, stream>>>(x, (const TD_*)delta, n_delta, stride, alpha, gain, eps, (TA_*)act, H); \
+        else postnorm_kernel<TA_, TD_><<<T, threads, 0, stream>>>(x, (const TD_*)delta, n_delta, stride, alpha, gain, eps, (TA_*)act, H); \
+    } while (0)
     const int dd = delta ? dt_d : QE_F32;
     if (dt_a == QE_F32 && dd == QE_F32) QE_PN(float, float);
     else if (dt_a == QE_BF16 && dd == QE_F32) QE_PN(bf16_t, float);
