@@ -196,3 +196,23 @@ def test_recorded_decode_steps_give_the_tokens_of_steps_run_as_they_come(folders
         if use_graphs:
             assert runner.graph_steps_of["decode"] == 10
     assert outs[0] == outs[1]
+
+
+def test_command_line_with_random_weights(tmp_path, capsys):
+    """main.py writes random weights for a Zarorax config.json and generates from token ids."""
+    import json
+    import main as cli
+    cfg, _, page = TINY["Q"]
+    cfg_path = tmp_path / "config.json"
+    cfg_path.write_text(json.dumps(cfg))
+    folder = str(tmp_path / "model")
+    rc = cli.main(["--model-name-or-path", folder, "--random-weights", str(cfg_path), "--seed", "3", "--prompt-ids", "5,17,3",
+                   "--prompt-ids", "9,9,200,41", "--max-new-tokens", "6", "--block-size", str(page), "--max-model-len", "64",
+                   "--ignore-eos", "--stats"])
+    assert rc == 0
+    out = capsys.readouterr().out
+    assert out.count("Prompt:") == 2 and "5 17 3" in out
+    stats = json.loads(out.strip().splitlines()[-1])
+    assert stats["graph_steps_decode"] >= 4                 # single new tokens were replayed from recorded steps
+    cfg_, w_ = Z.read_folder(folder)
+    assert set(w_) == set(random_tensors(cfg, 0))           # every tensor of the design, by its name

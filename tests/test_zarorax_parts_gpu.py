@@ -279,3 +279,21 @@ def test_latent_attention_on_the_matrix_units(R, Dr, H, P, lengths, new):
         worst = max(worst, rel(out[i], w @ keys[:, :R]))
     assert worst < 1.5e-2, worst
     assert rel(out, plain.double().cpu()) < 2e-2               # every row against the kernel on the vector units
+
+
+@pytest.mark.parametrize("taps", [2, 4])
+def test_short_convolution_of_single_rows_in_one_launch(taps):
+    """Steps in which every request brings one token: convolution and the state's shift in one launch give what
+    the two launches give, state included."""
+    H, B = 96, 5
+    g = torch.Generator().manual_seed(taps)
+    w = torch.randn(H, taps, generator=g).to(DEV)
+    xs = [torch.randn(B, H, generator=g).to(DEV) for _ in range(6)]
+    seq = torch.tensor([3, 0, 4, 1, 2], dtype=torch.int32, device=DEV)
+    a = torch.randn(6, taps - 1, H, generator=g).to(DEV)
+    b = a.clone()
+    for x in xs:
+        one = ops().short_conv(x, w, a, seq, torch.float32, single_rows=True)
+        two = ops().short_conv(x, w, b, seq, torch.float32)
+        assert torch.equal(one, two) and torch.equal(a, b)
+    assert torch.equal(a[3, -1], xs[-1][0]) and torch.equal(a[5], b[5])
