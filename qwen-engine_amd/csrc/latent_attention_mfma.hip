@@ -217,29 +217,34 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     }
 }
 
-// One wave per (token, head): the splits' partial results, in the order of the splits.  Lane s fetches split
-// s's maximum and sum, so that the weights are there after one trip to memory.
-__global__ __launch_bounds__(64) void latent_attention_merge_kernel(const float* __restrict__ part_acc,
-                                                                    const float* __restrict__ part_ml,
-                                                                    bf16_t* __restrict__ out, int NS, int R, int RP) {
+// One block per (token, head): the splits' partial results, in the order of the splits.  Lane s of the first
+// wave fetches split s's maximum and sum, so that the weights are there after one trip to memory; then every
+// thread adds up its output numbers, eight splits' loads at a time.
+__global__ __launch_bounds__(256) void latent_attention_merge_kernel(const float* __restrict__ part_acc,
+                                                                     const float* __restrict__ part_ml,
+                                                                     bf16_t* __restrict__ out, int NS, int R, int RP) {
     __shared__ float wgt[64];
+    __shared__ float inv_l;
     const long th = blockIdx.x;
-    const int lane = threadIdx.x;
-    const float* pm = part_ml + th * NS * 2;
-    const float ms = lane < NS ? pm[2 * lane] : -INFINITY;
-    const float ls = lane < NS ? pm[2 * lane + 1] : 0.f;
-    const float M = wave_max(ms);
-    const float w = ms == -INFINITY ? 0.f : __expf(ms - M);
-    wgt[lane] = w;
+    const int tid = threadIdx.x;
+    if (tid < 64) {
+        const float* pm = part_ml + th * NS * 2;
+        const float ms = tid < NS ? pm[2 * tid] : -INFINITY;
+        const float ls = tid < NS ? pm[2 * tid + 1] : 0.f;
+        const float M = wave_max(ms);
+        const float w = ms == -INFINITY ? 0.f : __expf(ms - M);
+        wgt[tid] = w;
+        float L = 0.f;
+        for (int s = 0; s < NS; ++s) L = fmaf(__shfl(w, s, 64), __shfl(ls, s, 64), L);      // in the order of the splits
+        if (tid == 0) inv_l = 1.f / L;
+    }
     __syncthreads();
-    float L = 0.f;
-    for (int s = 0; s < NS; ++s) L = fmaf(wgt[s], __shfl(ls, s, 64), L);      // in the order of the splits
-    const float inv = 1.f / L;
-    for (int d = lane; d < R; d += 64) {
+    const float inv = inv_l;
+    for (int d = tid; d < R; d += blockDim.x) {
         const float* pa = part_acc + th * NS * RP + d;
         float a = 0.f;
         int s = 0;
-        for (; s + 8 <= NS; s += 8) {                  // eight splits' loads together, added in the order of s
+        for (; s + 8 <= NS; s += 8) {
             float v[8];
 #pragma unroll
             for (int u = 0; u < 8; ++u) v[u] = pa[(long)(s + u) * RP];
@@ -277,7 +282,7 @@ static void latent_plan(int T, int H, int& TOK, int& HGB, int& NS) {
     NS = 1;
     if (blocks < 256) {
         NS = qe_cdiv(256, blocks);
-        int cap = T <= 64 ? 128 / T : 8;
+        int cap = T <= 64 ? 256 / T : 8;
         if (cap < 8) cap = 8;
         if (cap > 32) cap = 32;
         if (NS > cap) NS = cap;
@@ -333,7 +338,7 @@ extern "C" int qe_latent_attention_mfma(const void* qp, void* out, const void* c
 #undef QE_LA
     QE_LAUNCH_CHECK();
     if (NS > 1) {
-        latent_attention_merge_kernel<<<T * H, 64, 0, stream>>>(part_acc, part_ml, (bf16_t*)out, NS, R, (int)RP);
+        latent_attention_merge_kernel<<<T * H, R >= 256 ? 256 : (R >= 128 ? 128 : 64), 0, stream>>>(part_acc, part_ml, (bf16_t*)out, NS, R, (int)RP);
         QE_LAUNCH_CHECK();
     }
     return 0;

@@ -34,30 +34,6 @@ __global__ void short_conv_kernel(const float* __restrict__ x, const float* __re
     Elem<TA>::store(out + t * H + c, acc);
 }
 
-// Four channels a thread (H a multiple of 4): the rows and the state in 16-byte pieces.
-template <typename TA>
-__global__ void short_conv4_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                                   const float* __restrict__ state, const int* __restrict__ tok_seq,
-                                   TA* __restrict__ out, int T, int H, int taps) {
-    const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
-    const long t = blockIdx.y;
-    if (c >= H) return;
-    const int n1 = taps - 1;
-    const int s = tok_seq[t];
-    int before = 0;
-    while (before < n1 && t - 1 - before >= 0 && tok_seq[t - 1 - before] == s) ++before;
-    float acc[4];
-    Vec4<float>::load(x + t * H + c, acc);
-    for (int k = n1; k >= 0; --k) {                   // oldest input first, as in short_conv_kernel
-        float v[4];
-        if (k <= before) Vec4<float>::load(x + (t - k) * H + c, v);
-        else Vec4<float>::load(state + ((long)s * n1 + (n1 - k + before)) * H + c, v);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i] = fmaf(w[(long)(c + i) * taps + n1 - k], v[i], acc[i]);
-    }
-    Vec4<TA>::store(out + t * H + c, acc);
-}
-
 // After the convolution: the state takes the portion's last taps - 1 inputs.  A portion shorter than
 // that moves the state's old entries up first; its first row's thread does all of it, so that no
 // thread reads what another writes.
@@ -121,16 +97,7 @@ extern "C" int qe_short_conv(const float* x, const float* w, float* state, const
         QE_LAUNCH_CHECK();
         return 0;
     }
-    if (H % 4 == 0 && T > 16) {                       // many rows: bound by the bytes, four channels a thread
-        const int t4 = H / 4 >= 256 ? 256 : 64;
-        dim3 grid4(qe_cdiv(H / 4, t4), T);
-        if (dt_a == QE_F32)
-            short_conv4_kernel<float><<<grid4, t4, 0, stream>>>(x, w, state, tok_seq, (float*)out, T, H, taps);
-        else if (dt_a == QE_BF16)
-            short_conv4_kernel<bf16_t><<<grid4, t4, 0, stream>>>(x, w, state, tok_seq, (bf16_t*)out, T, H, taps);
-        else
-            QE_REQUIRE(false, "short_conv: unknown output type %d", dt_a);
-    } else if (dt_a == QE_F32)
+    if (dt_a == QE_F32)
         short_conv_kernel<float><<<grid, threads, 0, stream>>>(x, w, state, tok_seq, (float*)out, T, H, taps);
     else if (dt_a == QE_BF16)
         short_conv_kernel<bf16_t><<<grid, threads, 0, stream>>>(x, w, state, tok_seq, (bf16_t*)out, T, H, taps);
