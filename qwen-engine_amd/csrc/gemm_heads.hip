@@ -92,56 +92,69 @@ extern "C" int qe_gemm_heads(const void* x, long xs_t, long xs_h, const void* w,
 // ---- the same on the matrix units (bfloat16, K a multiple of 8) -----------------------------------------------
 // out^T[n][t] = sum_k W_h[n][k] x[t][h][k] by v_mfma_f32_16x16x32_bf16: the head's weight rows are the A operand,
 // the tokens' rows the B operand, both read straight from memory in 16-byte pieces.  A block's four waves take
-// 16 output features each for MT * 16 tokens; blockIdx.z is the head.
+// NT * 16 output features each for MT * 16 tokens; blockIdx.z is the head.
 typedef __attribute__((ext_vector_type(8))) __bf16 gh_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float gh_floatx4;
 
-template <int MT>
+template <int MT, int NT>
 __global__ __launch_bounds__(256) void gemm_heads_mfma_kernel(
     const bf16_t* __restrict__ x, long xs_t, long xs_h, const bf16_t* __restrict__ w, bf16_t* __restrict__ out, long os_t,
     long os_h, const bf16_t* __restrict__ gate, int T, int N, int K) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, nn = lane & 15;
     const int h = blockIdx.z, H = gridDim.z;
-    const int n_base = blockIdx.x * 64 + wave * 16;
+    const int n_base = blockIdx.x * 64 * NT + wave * 16 * NT;      // a wave takes NT groups of 16 features
     if (n_base >= N) return;
     const int t_base = blockIdx.y * MT * 16;
-    const int n_row = n_base + nn < N ? n_base + nn : N - 1;
-    const bf16_t* wr = w + ((long)h * N + n_row) * K + g * 8;
+    const bf16_t* wr[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        const int n_row = n_base + j * 16 + nn < N ? n_base + j * 16 + nn : N - 1;
+        wr[j] = w + ((long)h * N + n_row) * K + g * 8;
+    }
     const bf16_t* xr[MT];
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
         const int t = t_base + i * 16 + nn;
         xr[i] = x + (long)(t < T ? t : T - 1) * xs_t + h * xs_h + g * 8;
     }
-    gh_floatx4 acc[MT];
+    gh_floatx4 acc[NT][MT];
 #pragma unroll
-    for (int i = 0; i < MT; ++i) acc[i] = gh_floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int i = 0; i < MT; ++i) acc[j][i] = gh_floatx4{0.f, 0.f, 0.f, 0.f};
     const gh_bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll 2
     for (int k0 = 0; k0 < K; k0 += 32) {
         const bool kin = k0 + g * 8 < K;
-        const gh_bf16x8 a = kin ? *(const gh_bf16x8*)(wr + k0) : zero8;
+        gh_bf16x8 a[NT], b[MT];
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            const gh_bf16x8 b = kin ? *(const gh_bf16x8*)(xr[i] + k0) : zero8;
-            acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[i], 0, 0, 0);
-        }
+        for (int j = 0; j < NT; ++j) a[j] = kin ? *(const gh_bf16x8*)(wr[j] + k0) : zero8;
+#pragma unroll
+        for (int i = 0; i < MT; ++i) b[i] = kin ? *(const gh_bf16x8*)(xr[i] + k0) : zero8;
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int i = 0; i < MT; ++i) acc[j][i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[i], acc[j][i], 0, 0, 0);
     }
-    const int n0 = n_base + g * 4;     // lane (g, nn) holds token t_base + i * 16 + nn at the features n0 .. n0 + 3
+    // lane (g, nn) holds token t_base + i * 16 + nn at the features n_base + j * 16 + g * 4 .. + 3
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
         const int t = t_base + i * 16 + nn;
         if (t >= T) continue;
-        bf16_t* o = out + (long)t * os_t + h * os_h + n0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            if (n0 + j >= N) break;
-            float v = acc[i][j];
-            if (gate) {
-                const float gv = Elem<bf16_t>::load(gate + ((long)t * H + h) * N + n0 + j);
-                v = v / (1.f + __expf(-gv));
+        for (int j = 0; j < NT; ++j) {
+            const int n0 = n_base + j * 16 + g * 4;
+            bf16_t* o = out + (long)t * os_t + h * os_h + n0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (n0 + e >= N) break;
+                float v = acc[j][i][e];
+                if (gate) {
+                    const float gv = Elem<bf16_t>::load(gate + ((long)t * H + h) * N + n0 + e);
+                    v = v / (1.f + __expf(-gv));
+                }
+                Elem<bf16_t>::store(o + e, v);
             }
-            Elem<bf16_t>::store(o + j, v);
         }
     }
 }
@@ -155,12 +168,13 @@ extern "C" int qe_gemm_heads_mfma(const void* x, long xs_t, long xs_h, const voi
     if (T == 0) return 0;
     if (T <= 32) {
         dim3 grid(qe_cdiv(N, 64), qe_cdiv(T, 16), H);
-        gemm_heads_mfma_kernel<1><<<grid, 256, 0, stream>>>((const bf16_t*)x, xs_t, xs_h, (const bf16_t*)w, (bf16_t*)out,
+        gemm_heads_mfma_kernel<1, 1><<<grid, 256, 0, stream>>>((const bf16_t*)x, xs_t, xs_h, (const bf16_t*)w, (bf16_t*)out,
                                                              os_t, os_h, (const bf16_t*)gate, T, N, K);
     } else {
         QE_REQUIRE(qe_cdiv(T, 64) <= 65535, "gemm_heads (mfma): too many rows");
-        dim3 grid(qe_cdiv(N, 64), qe_cdiv(T, 64), H);
-        gemm_heads_mfma_kernel<4><<<grid, 256, 0, stream>>>((const bf16_t*)x, xs_t, xs_h, (const bf16_t*)w, (bf16_t*)out,
+        // (many rows: a wave takes 32 features for 64 tokens, six loads for eight products)
+        dim3 grid(qe_cdiv(N, 128), qe_cdiv(T, 64), H);
+        gemm_heads_mfma_kernel<4, 2><<<grid, 256, 0, stream>>>((const bf16_t*)x, xs_t, xs_h, (const bf16_t*)w, (bf16_t*)out,
                                                              os_t, os_h, (const bf16_t*)gate, T, N, K);
     }
     QE_LAUNCH_CHECK();

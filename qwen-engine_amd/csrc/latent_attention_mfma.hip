@@ -1,5 +1,5 @@
 // Attention over one cached latent per token on the matrix units (bfloat16), for prompts' portions and
-// for single new tokens alike.  See latent_attention.hip for the contract: packed queries
+// for single new tokens alike.  See latent_attention.hip for what goes in and out: packed queries
 // qp [T, H, R + Dr], cache rows [R + Dr] of which the first R are also the value, out [T, H, R].
 //
 // All heads read the same rows, so a wave's 16 columns are 16 heads of one token, and a block's four waves

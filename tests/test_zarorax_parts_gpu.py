@@ -134,7 +134,7 @@ def _latent_case(dtype, R, Dr, H, P, lengths, seed, stand_out=None):
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 3e-6), (torch.bfloat16, 1e-2)])
-@pytest.mark.parametrize("R,Dr,H,P", [(40, 8, 3, 8), (64, 64, 1, 16), (128, 32, 16, 4)])
+@pytest.mark.parametrize("R,Dr,H,P", [(40, 8, 3, 8), (64, 64, 1, 16), (96, 32, 16, 4)])
 def test_latent_attention_over_pages(dtype, tol, R, Dr, H, P):
     lengths = [3 * P + 1, 1, 64, 65, 5 * P]
     cache, table, rows = _latent_case(dtype, R, Dr, H, P, lengths, seed=R + H)
@@ -250,7 +250,7 @@ def test_experts_over_rows_grouped_on_the_device(dtype, tol, T, H, Fd):
     (512, 64, 16, 16, [300, 1, 77], [300, 1, 77]),        # whole prompts side by side, many rows: tokens share a block
     (512, 64, 16, 16, [700, 33, 64, 65, 129], [1, 1, 1, 1, 1]),   # single new tokens: the keys are cut into splits
     (256, 32, 128, 8, [90, 200], [3, 70]),                # many heads: several head groups per token
-    (128, 32, 5, 16, [40, 41, 260], [40, 2, 100]),        # fewer heads than a wave has columns; mixed step
+    (160, 32, 5, 16, [40, 41, 260], [40, 2, 100]),        # fewer heads than a wave has columns; mixed step
     (64, 0, 24, 4, [130, 19], [130, 1]),                  # no rotated part; heads that fill one group and half of the next
     (200, 24, 8, 32, [150], [150]),                       # sizes that are no multiple of 16 or 32
 ])

@@ -43,9 +43,9 @@ ZQ = {
          "mlp": {"kind": "moe", "expert": {"ff": 64, "limit": 2.0},
                  "router": {"experts": 4, "top": 1, "groups": {"count": 1, "keep": 1}}}},
         {"type": "latent_attention",
-         "mixer": {"heads": 4, "dim": 32, "rot_dim": 32, "vdim": 32, "kv_rank": 128, "q_rank": 64, "scale": 0.12,
-                   "rot": {"base": 100000.0, "dims": 32}},
-         "mlp": {"kind": "moe", "expert": {"ff": 96, "limit": 1.0},
+         "mixer": {"heads": 4, "dim": 16, "rot_dim": 16, "vdim": 16, "kv_rank": 96, "q_rank": 64, "scale": 0.17,
+                   "rot": {"base": 100000.0, "dims": 16}},
+         "mlp": {"kind": "moe", "expert": {"ff": 160, "limit": 1.0},
                  "router": {"experts": 8, "top": 3, "groups": {"count": 4, "keep": 4}}}},
     ],
 }
