@@ -216,3 +216,68 @@ def test_command_line_with_random_weights(tmp_path, capsys):
     assert stats["graph_steps_decode"] >= 4                 # single new tokens were replayed from recorded steps
     cfg_, w_ = Z.read_folder(folder)
     assert set(w_) == set(random_tensors(cfg, 0))           # every tensor of the design, by its name
+
+
+# Sizes at which the bfloat16 mode runs the kernels on the matrix units inside the engine: latents that fill several
+# blocks of 16, heads that do not fill a wave's 16 columns or spill into a second group, enough (token, choice) pairs in
+# a long prompt for the tiled grouped product, prompts long enough for several key splits and for blocks of four tokens.
+ZM = {
+    "architecture": "Zarorax", "vocab": 701, "width": 320, "postln_alpha": 2.5, "norm": {"eps": 1e-5},
+    "canon": {"taps": 3},
+    "layers": [
+        {"type": "latent_attention",
+         "mixer": {"heads": 6, "dim": 40, "rot_dim": 24, "vdim": 48, "kv_rank": 104, "q_rank": 72, "scale": 0.11,
+                   "rot": {"base": 20000.0, "dims": 24}},
+         "mlp": {"kind": "dense", "ff": 448}},
+        {"type": "latent_attention_2",
+         "mixer": {"heads": 20, "dim": 24, "rot_dim": 8, "vdim": 16, "kv_rank": 200, "scale": 0.14,
+                   "rot": {"base": 3000.0, "dims": 8}},
+         "mlp": {"kind": "moe", "expert": {"ff": 64, "limit": 1.2},
+                 "router": {"experts": 12, "top": 3, "groups": {"count": 3, "keep": 2}}}},
+        {"type": "latent_attention_2",
+         "mixer": {"heads": 20, "dim": 24, "rot_dim": 8, "vdim": 16, "kv_rank": 200, "scale": 0.14,
+                   "rot": {"base": 3000.0, "dims": 8}},
+         "mlp": {"kind": "moe", "expert": {"ff": 64, "limit": 1.2},
+                 "router": {"experts": 12, "top": 3, "groups": {"count": 3, "keep": 2}}}, "weights_of": 1},
+    ],
+}
+
+
+@pytest.fixture(scope="module")
+def medium(tmp_path_factory):
+    folder = write_folder(str(tmp_path_factory.mktemp("zarorax_m") / "model"), ZM, random_tensors(ZM, 21))
+    reqs = _requests(ZM["vocab"], (610, 75, 380), seed=14)
+    return folder, reqs, _reference(folder, reqs)
+
+
+def _medium_mixed(reqs):
+    """The long prompt in large portions beside the others' small portions and single tokens."""
+    t = traces.Trace()
+    a, b, c = reqs["q0"], reqs["q1"], reqs["q2"]
+    t.step([("q0", a[:400]), ("q1", b[:3])])
+    t.step([("q1", b[3:4]), ("q0", a[400:590]), ("q2", c[:350])])
+    t.step([("q2", c[350:352]), ("q1", b[4:5])])
+    for i in range(20):
+        entries = [("q0", a[590 + i:591 + i]), ("q2", c[352 + i:353 + i])]
+        if 5 + i < len(b):
+            entries.append(("q1", b[5 + i:6 + i]))
+        t.step(entries)
+    t.step([("q1", b[25:]), ("q2", c[372:])], end=["q0", "q1", "q2"])
+    return t
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["whole", "mixed"])
+def test_medium_sizes_with_long_prompts(medium, tmp_path, dtype, cut):
+    folder, reqs, ref = medium
+    trace = traces.whole(reqs) if cut == "whole" else _medium_mixed(reqs)
+    out = str(tmp_path / "out")
+    traces.run_in_process(trace, folder, dtype, out, 16)
+    got = traces.collect(trace, out, ZM["vocab"])
+    if cut == "mixed":
+        ref = {rid: rows[:max(got[rid]) + 1] for rid, rows in ref.items()}
+    if dtype == "float32":
+        bad, worst = traces.first_mismatch(got, ref, 2e-4)
+        assert bad is None, f"first wrong logits at (request, position, relative error) {bad}"
+    else:
+        _assert_close_but_for_close_calls(got, ref, f"{cut} against the plain model")
