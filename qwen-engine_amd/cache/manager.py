@@ -43,8 +43,10 @@ class OutOfPages(CacheError):
 @dataclass(frozen=True)
 class GroupSpec:
     """The need of a group of layers: ``window`` None keeps every key, an int
-    keeps the ``window`` most recent positions (the current one included)."""
+    keeps the ``window`` most recent positions (the current one included) and, with
+    ``keep_first``, the request's first ``keep_first`` positions as well."""
     window: Optional[int] = None
+    keep_first: int = 0
 
 
 class PagePool:
@@ -196,6 +198,8 @@ class CacheManager:
         for g in self.groups:
             if g.window is not None and g.window <= 0:
                 raise CacheError("a window must be positive")
+            if g.keep_first < 0:
+                raise CacheError("keep_first must not be negative")
         self.page_size = page_size
         self.pools = [PagePool(n, scatter=scatter_pages) for n in num_pages]
         self.slots = StateSlots(max_requests)
@@ -267,6 +271,13 @@ class CacheManager:
             return 0
         first_key = max(0, next_pos - w + 1)
         return first_key // self.page_size
+
+    def kept_first_pages(self, g: int) -> int:
+        """Pages at a request's start that a group with a window holds for good: those of its kept first positions."""
+        grp = self.groups[g]
+        if grp.window is None or grp.keep_first <= 0:
+            return 0
+        return (grp.keep_first + self.page_size - 1) // self.page_size
 
     def pages_needed(self, req_id: Hashable, new_len: int) -> List[int]:
         """New pages per group for the request to hold positions up to new_len - 1,
@@ -360,7 +371,8 @@ class CacheManager:
             if self.groups[g].window is None:
                 continue
             live_from = min(self._first_live_page(g, new_len), len(table))
-            for i in range(rc.released[g], live_from):   # pages below rc.released[g] went back earlier
+            kept = self.kept_first_pages(g)                # (the pages of the kept first positions never go back)
+            for i in range(max(rc.released[g], kept), live_from):   # pages below rc.released[g] went back earlier
                 if table[i] >= 0:
                     self._release(g, table[i])
                     table[i] = -1

@@ -12,11 +12,13 @@ from .manager import GroupSpec
 class KVNeed:
     """Keys and values of every position (window None) or of the last ``window``.  ``planes``: 2 for a
     key and a value tile per head and page; 1 for a part that keeps one row per token (a latent from
-    which it forms both)."""
+    which it forms both).  ``keep_first``: with a window, the request's first keys that stay seen, and so
+    stay held, wherever the window stands."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     planes: int = 2
+    keep_first: int = 0
 
 
 @dataclass(frozen=True)
@@ -75,7 +77,7 @@ def plan_cache(entry_needs: Sequence[tuple]) -> CachePlan:
                     raise ValueError(f"schedule entry {i} cannot read the cache of entry {cache_from}: "
                                      f"their key/value shapes differ")
                 if kv is not None and src_kv is not None and src_kv.window is not None and \
-                        (kv.window is None or kv.window > src_kv.window):
+                        (kv.window is None or kv.window > src_kv.window or kv.keep_first > src_kv.keep_first):
                     # the source's group gives pages back once its own window has passed them: a reader
                     # that looks further back would read pages that are no longer the request's
                     raise ValueError(f"schedule entry {i} (window {kv.window}) cannot read the cache of entry "
@@ -89,7 +91,7 @@ def plan_cache(entry_needs: Sequence[tuple]) -> CachePlan:
                 user_source.append(None)
                 user_group.append(None)
                 continue
-            spec = GroupSpec(window=kv.window)
+            spec = GroupSpec(window=kv.window, keep_first=kv.keep_first if kv.window is not None else 0)
             if spec not in groups:
                 groups.append(spec)
             user_kv.append(kv)

@@ -55,3 +55,11 @@ def _zarorax(d):
 
 
 register_architecture("Zarorax", _zarorax)
+
+
+def _nufavik(d):
+    from .nufavik import NufavikConfig
+    return NufavikConfig.from_dict(d)
+
+
+register_architecture("Nufavik", _nufavik)

@@ -151,6 +151,85 @@ class PostNormLayerSpec:
 
 
 @dataclass(frozen=True)
+class RopeHalfAnglesSpec:
+    """Half-split rotation of the first ``rotary_dim`` numbers of a head (number i < rotary_dim / 2 pairs with
+    i + rotary_dim / 2) by ``position * theta ** (-2 i / rotary_dim)``; the rest of the head passes unchanged.
+    The kernels form angle, sine and cosine in 32-bit from the frequencies: no table, no limit of positions."""
+    theta: float
+    rotary_dim: int
+    kind: str = "rope_half_angles"
+
+
+@dataclass(frozen=True)
+class ConvAttentionSpec:
+    """Grouped-query attention whose projected queries, keys and values (with biases if ``qkv_bias``) each pass
+    a causal convolution of ``conv_taps`` taps over time on every channel before q and k are rotated.  Keys have
+    ``head_dim`` numbers, values ``v_head_dim``.  ``window`` None: all earlier keys; else the last ``window`` keys
+    (the query's own included) and, wherever the window stands, the request's first ``keep_first`` keys.
+    ``sink``: the softmax's denominator has a 1 added (one more entry of score 0 that carries no value).
+    ``names``: the tensors' names inside the part for q, k, v and the output projection; a bias is the
+    projection's name + ``bias_suffix``, a convolution's weights [channels, taps] its name + ``conv_suffix``."""
+    num_heads: int
+    num_kv_heads: int
+    head_dim: int
+    v_head_dim: int
+    scale: float
+    conv_taps: int = 1
+    qkv_bias: bool = False
+    window: Optional[int] = None
+    keep_first: int = 0
+    sink: bool = False
+    position: Optional[object] = None
+    names: Tuple[str, str, str, str] = ("q", "k", "v", "o")
+    bias_suffix: str = ".b"
+    conv_suffix: str = ".conv"
+    kind: str = "conv_attention"
+
+
+@dataclass(frozen=True)
+class BiasedMoESpec:
+    """A routed mixture of small feed-forwards down(relu(up x)^2) without biases.  Scores: softmax of the
+    router's 32-bit logits over ``num_experts + num_identity`` outputs; the ``top`` largest of score + correction
+    (a tensor of the layer) are chosen; their weights are their scores without the correction, divided by their
+    sum (+ 1e-20), times ``route_scale``.  The last ``num_identity`` outputs are identity experts: their output is
+    the input itself, and they have no tensors."""
+    num_experts: int
+    num_identity: int
+    top: int
+    intermediate_size: int
+    route_scale: float
+    kind: str = "biased_moe"
+
+
+@dataclass(frozen=True)
+class ParallelLayerSpec:
+    """One block with a single norm whose output both branches read: n = norm(x); x <- x + (mixer(n) + ffn(n)).
+    ``ffn`` may be None.  ``names``: the checkpoint names inside ``prefix`` of norm, mixer and feed-forward; a
+    norm that is one tensor carries the norm's name itself."""
+    prefix: str
+    norm: object
+    mixer: object
+    ffn: Optional[object]
+    names: Tuple[str, str, str] = ("norm1", "mix", "mlp")
+    kind: str = "parallel_block"
+
+
+@dataclass(frozen=True)
+class BareRMSNormSpec:
+    """RMSNorm whose weight tensor carries the part's own name (no ``.weight`` behind it)."""
+    eps: float
+    kind: str = "rmsnorm_bare"
+
+
+@dataclass(frozen=True)
+class StreamScaleSpec:
+    """The stream right after the embedding is multiplied by ``scale`` (in 32-bit); no tensors."""
+    scale: float
+    prefix: str = ""
+    kind: str = "stream_scale"
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     """One pre-norm residual block: x += mixer(norm(x)); x += ffn(norm(x)).
 

@@ -9,20 +9,21 @@
 
 int qe_attention_generic(const void* q, void* out, const void* cache, const int* positions,
                          const int* tok_seq, const int* block_table, int max_blocks, const int* tokens,
-                         int T, int Hq, int Hkv, int D, int P, float scale, int window, int dt_a,
-                         hipStream_t stream);
+                         int T, int Hq, int Hkv, int D, int P, float scale, int window, int keep_first, int sink,
+                         int dt_a, hipStream_t stream);
 bool qe_attention_decode_ok(int Hq, int Hkv, int D, int P, int dt_a);
 size_t qe_attention_decode_workspace(int n_dec, int Hq, int D, int num_splits);
 int qe_attention_decode(const void* q, void* out, const void* cache, const int* dec_tokens, int n_dec,
                         const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
-                        const int* shared_keys, int Hq, int Hkv, int D, int P, float scale, int window, int max_position,
-                        int split_keys, void* workspace, size_t workspace_bytes, hipStream_t stream);
+                        const int* shared_keys, int Hq, int Hkv, int D, int P, float scale, int window, int keep_first,
+                        int sink, int max_position, int split_keys, void* workspace, size_t workspace_bytes,
+                        hipStream_t stream);
 
 int qe_attention_prefill(const void* q, void* out, const void* cache, const int* tiles, int num_tiles,
                          const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
                          int Hq, int Hkv, int D, int P, float scale, int window, int groups,
                          int seg_keys, int max_keys, int keys_row, void* workspace, size_t workspace_bytes,
-                         hipStream_t stream);
+                         hipStream_t stream, int keep_first = 0, int sink = 0);
 int qe_attention_prefill_segment_keys(long blocks, int max_keys);
 int qe_attention_prefill_segments(long blocks);
 int qe_attention_prefill_uncut_keys();
@@ -87,26 +88,28 @@ extern "C" long qe_attention_prefill_workspace_bytes_for(int num_tiles, int Hq, 
 extern "C" int qe_attention_prefill_run(const void* q, void* out, const void* cache, const int* tiles,
                                         int num_tiles, const int* positions, const int* tok_seq,
                                         const int* block_table, int max_blocks, int Hq, int Hkv, int D, int P,
-                                        float scale, int window, int groups, int seg_keys, int max_keys,
-                                        int keys_row, void* workspace, long workspace_bytes, hipStream_t stream) {
-    QE_REQUIRE(num_tiles >= 0 && Hq > 0 && Hkv > 0 && max_blocks > 0 && window >= 0 && workspace_bytes >= 0,
-               "prefill attention: bad sizes");
+                                        float scale, int window, int keep_first, int sink, int groups, int seg_keys,
+                                        int max_keys, int keys_row, void* workspace, long workspace_bytes,
+                                        hipStream_t stream) {
+    QE_REQUIRE(num_tiles >= 0 && Hq > 0 && Hkv > 0 && max_blocks > 0 && window >= 0 && keep_first >= 0 &&
+               workspace_bytes >= 0, "prefill attention: bad sizes");
     return qe_attention_prefill(q, out, cache, tiles, num_tiles, positions, tok_seq, block_table, max_blocks,
                                 Hq, Hkv, D, P, scale, window, groups, seg_keys, max_keys, keys_row, workspace,
-                                (size_t)workspace_bytes, stream);
+                                (size_t)workspace_bytes, stream, keep_first, sink);
 }
 
-// tokens: null for all T rows of q, else n_tokens row indices.
+// tokens: null for all T rows of q, else n_tokens row indices.  keep_first: the first keys of a request
+// that every later query sees wherever its window stands; sink: a 1 is added to the softmax's denominator.
 extern "C" int qe_attention(const void* q, void* out, const void* cache, const int* positions,
                             const int* tok_seq, const int* block_table, int max_blocks, const int* tokens,
-                            int n_tokens, int Hq, int Hkv, int D, int P, float scale, int window, int dt_a,
-                            hipStream_t stream) {
+                            int n_tokens, int Hq, int Hkv, int D, int P, float scale, int window, int keep_first,
+                            int sink, int dt_a, hipStream_t stream) {
     QE_REQUIRE(n_tokens >= 0 && Hq > 0 && Hkv > 0 && D > 0 && P > 0 && max_blocks > 0, "attention: bad sizes");
     QE_REQUIRE(Hq % Hkv == 0, "attention: %d query heads are no multiple of %d key/value heads", Hq, Hkv);
-    QE_REQUIRE(window >= 0, "attention: negative window");
+    QE_REQUIRE(window >= 0 && keep_first >= 0, "attention: negative window or kept keys");
     if (n_tokens == 0) return 0;
     return qe_attention_generic(q, out, cache, positions, tok_seq, block_table, max_blocks, tokens, n_tokens,
-                                Hq, Hkv, D, P, scale, window, dt_a, stream);
+                                Hq, Hkv, D, P, scale, window, keep_first, sink, dt_a, stream);
 }
 
 extern "C" int qe_attention_decode_supported(int Hq, int Hkv, int D, int P, int dt_a) {
@@ -150,11 +153,12 @@ extern "C" int qe_attention_decode_fused_run(const void* qkv, void* out, void* c
 extern "C" int qe_attention_decode_run(const void* q, void* out, const void* cache, const int* dec_tokens,
                                        int n_dec, const int* positions, const int* tok_seq,
                                        const int* block_table, int max_blocks, const int* shared_keys,
-                                       int Hq, int Hkv, int D, int P, float scale, int window,
+                                       int Hq, int Hkv, int D, int P, float scale, int window, int keep_first, int sink,
                                        int max_position, int split_keys, void* workspace, long workspace_bytes,
                                        hipStream_t stream) {
-    QE_REQUIRE(Hq > 0 && Hkv > 0 && max_blocks > 0 && window >= 0 && max_position >= 0, "decode attention: bad sizes");
+    QE_REQUIRE(Hq > 0 && Hkv > 0 && max_blocks > 0 && window >= 0 && keep_first >= 0 && max_position >= 0,
+               "decode attention: bad sizes");
     return qe_attention_decode(q, out, cache, dec_tokens, n_dec, positions, tok_seq, block_table, max_blocks,
-                               shared_keys, Hq, Hkv, D, P, scale, window, max_position, split_keys, workspace,
-                               (size_t)workspace_bytes, stream);
+                               shared_keys, Hq, Hkv, D, P, scale, window, keep_first, sink, max_position, split_keys,
+                               workspace, (size_t)workspace_bytes, stream);
 }

@@ -18,7 +18,7 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
     const int* __restrict__ dec_tokens, const int* __restrict__ positions, const int* __restrict__ tok_seq,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ shared_keys,
     float* __restrict__ part_acc, float* __restrict__ part_ml,
-    int Hq, int Hkv, int P, float scale, int window, int num_splits) {
+    int Hq, int Hkv, int P, float scale, int window, int keep_first, int num_splits) {
     constexpr int TILES = SPLIT / 16;
     const int lane = threadIdx.x, g = lane >> 4, n = lane & 15;
     const int split = blockIdx.x, kvh = blockIdx.y, di = blockIdx.z;
@@ -28,11 +28,14 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int k_begin = max(split * SPLIT, lo);
     const int k_end = min((split + 1) * SPLIT, p + 1);
+    // the request's kept first keys that lie behind the window, as far as they are this split's: [split * SPLIT, kf)
+    const int kf = min(min(keep_first, lo), (split + 1) * SPLIT);
+    const int first_tiles = kf > split * SPLIT ? (kf - split * SPLIT + 15) / 16 : 0;
     const int head = kvh * G + n;
     const bool head_ok = n < G;
     float* pacc = part_acc + (((long)di * Hq + head) * num_splits + split) * D;
     float* pml = part_ml + (((long)di * Hq + head) * num_splits + split) * 2;
-    if (k_begin >= k_end) {   // nothing of this split is seen by the token
+    if (k_begin >= k_end && first_tiles == 0) {   // nothing of this split is seen by the token
         if (head_ok && g == 0) { pml[0] = -INFINITY; pml[1] = 0.f; }
         return;
     }
@@ -41,12 +44,16 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
     // (keys that other requests read too are left in the caches, the others stream: see load_tile)
     const bool stream = !(shared_keys && split * SPLIT < shared_keys[row]);
     const long page_stride = 2L * Hkv * P * D;
-    const int tile0 = (k_begin - split * SPLIT) / 16;                 // first and one-past-last tile of the split
-    const int tile1 = (k_end - split * SPLIT + 15) / 16;
+    // the split's tiles that are walked: first_tiles from its start (kept first keys), then, from the window's
+    // first tile on, tile0 .. tile1 - 1 (tiles between the two are not read: their pages may have gone back)
+    const int tile1 = k_begin < k_end ? (k_end - split * SPLIT + 15) / 16 : first_tiles;
+    const int tile0 = k_begin < k_end ? max((k_begin - split * SPLIT) / 16, first_tiles) : first_tiles;
+    const int walk0 = first_tiles > 0 ? 0 : tile0;                    // first tile of the walk
+    const int gap = first_tiles > 0 ? tile0 - first_tiles : 0;        // tiles left out behind the first ones
     // lane i holds the page of tile i (one vector load for the whole split); a tile's page is
     // then read from that lane
     int my_page = 0;
-    if (lane >= tile0 && lane < tile1) my_page = bt[(split * SPLIT + lane * 16) / P];
+    if ((lane >= tile0 && lane < tile1) || lane < first_tiles) my_page = bt[(split * SPLIT + lane * 16) / P];
 
     bf16x8 qreg[D / 32];
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -59,22 +66,26 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
 
     // Two tile buffers used in turn: the loads of the next tile are issued before the current
     // one is computed, and nothing is copied from one buffer to the other.
-#define LOAD(buf_, i_) load_tile<D>(buf_, cache, __builtin_amdgcn_readlane(my_page, (i_)), page_stride, kvh, Hkv, P, \
-                                    (split * SPLIT + (i_) * 16) % P, g, n, stream)
-#define STEP(buf_, i_) attn_tile_step<D>(st, buf_, qreg, scale, split * SPLIT + (i_) * 16, g, k_begin, k_end, k_begin, k_end)
+    // (i_ counts the walk's tiles; TILE_OF: the tile of the split behind it)
+#define TILE_OF(i_) ((i_) < first_tiles ? (i_) : (i_) + gap)
+#define LOAD(buf_, i_) load_tile<D>(buf_, cache, __builtin_amdgcn_readlane(my_page, TILE_OF(i_)), page_stride, kvh, Hkv, P, \
+                                    (split * SPLIT + TILE_OF(i_) * 16) % P, g, n, stream)
+#define STEP(buf_, i_) attn_tile_step<D>(st, buf_, qreg, scale, split * SPLIT + TILE_OF(i_) * 16, g, k_begin, k_end, k_begin, k_end, kf)
     KVTile<D> ta, tb;
-    int i = tile0;
+    int i = walk0;
+    const int walk1 = tile1 - gap;
     LOAD(ta, i);
     while (true) {
-        if (i + 1 < tile1) LOAD(tb, i + 1);
+        if (i + 1 < walk1) LOAD(tb, i + 1);
         STEP(ta, i);
-        if (++i >= tile1) break;
-        if (i + 1 < tile1) LOAD(ta, i + 1);
+        if (++i >= walk1) break;
+        if (i + 1 < walk1) LOAD(ta, i + 1);
         STEP(tb, i);
-        if (++i >= tile1) break;
+        if (++i >= walk1) break;
     }
 #undef LOAD
 #undef STEP
+#undef TILE_OF
     float l = st.l;
     const float m = st.m;
     l += __shfl_xor(l, 16, 64);
@@ -321,7 +332,7 @@ __global__ __launch_bounds__(64) void attention_decode_fused_split_kernel(
 template <int D>
 __global__ __launch_bounds__(256) void attention_decode_merge_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml, const int* __restrict__ dec_tokens,
-    bf16_t* __restrict__ out, int Hq, int num_splits) {
+    bf16_t* __restrict__ out, int Hq, int num_splits, int sink) {
     constexpr int PER = (D + 63) / 64;
     __shared__ float red_o[4][D];
     __shared__ float red_l[4];
@@ -359,7 +370,8 @@ __global__ __launch_bounds__(256) void attention_decode_merge_kernel(
                 a[k][i] = d < D ? pacc[(long)(s < num_splits ? s : num_splits - 1) * D + d] : 0.f;
             }
         }
-        if (!reduced) { M = wave_max(M); reduced = true; }
+        // (sink: one more entry of score 0 that carries no value)
+        if (!reduced) { M = wave_max(M); if (sink) M = fmaxf(M, 0.f); reduced = true; }
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
             if (ms[k] == -INFINITY) continue;
@@ -377,7 +389,7 @@ __global__ __launch_bounds__(256) void attention_decode_merge_kernel(
     if (lane == 0) red_l[wave] = denom;
     __syncthreads();
     if (wave == 0) {
-        const float inv = 1.f / (red_l[0] + red_l[1] + red_l[2] + red_l[3]);
+        const float inv = 1.f / (red_l[0] + red_l[1] + red_l[2] + red_l[3] + (sink ? __expf(-M) : 0.f));
         bf16_t* orow = out + ((long)(dec_tokens ? dec_tokens[di] : di) * Hq + head) * D;
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
@@ -404,8 +416,9 @@ size_t qe_attention_decode_workspace(int n_dec, int Hq, int D, int num_splits) {
 // hold together): a hint for the caches, results do not depend on it.
 int qe_attention_decode(const void* q, void* out, const void* cache, const int* dec_tokens, int n_dec,
                         const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
-                        const int* shared_keys, int Hq, int Hkv, int D, int P, float scale, int window, int max_position,
-                        int split_keys, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+                        const int* shared_keys, int Hq, int Hkv, int D, int P, float scale, int window, int keep_first,
+                        int sink, int max_position, int split_keys, void* workspace, size_t workspace_bytes,
+                        hipStream_t stream) {
     QE_REQUIRE(qe_attention_decode_ok(Hq, Hkv, D, P, QE_BF16), "decode attention: sizes not taken");
     QE_REQUIRE(split_keys == 128 || split_keys == 256, "decode attention: splits of 128 or 256 keys, not %d", split_keys);
     if (n_dec == 0) return 0;
@@ -422,9 +435,9 @@ int qe_attention_decode(const void* q, void* out, const void* cache, const int* 
     do {                                                                                                \
         attention_decode_split_kernel<D_, S_><<<grid, 64, 0, stream>>>(                                 \
             (const bf16_t*)q, (const bf16_t*)cache, dec_tokens, positions, tok_seq, block_table,        \
-            max_blocks, shared_keys, part_acc, part_ml, Hq, Hkv, P, scale, window, num_splits);         \
+            max_blocks, shared_keys, part_acc, part_ml, Hq, Hkv, P, scale, window, keep_first, num_splits); \
         attention_decode_merge_kernel<D_><<<mgrid, 256, 0, stream>>>(part_acc, part_ml, dec_tokens,     \
-                                                                     (bf16_t*)out, Hq, num_splits);     \
+                                                                     (bf16_t*)out, Hq, num_splits, sink); \
     } while (0)
     if (D == 128 && split_keys == 128) QE_DECODE(128, 128);
     else if (D == 128) QE_DECODE(128, 256);
@@ -469,7 +482,7 @@ int qe_attention_decode_fused(const void* qkv, void* out, void* cache, const int
             shared_keys, slots, q_w, k_w, eps, table, part_acc, part_ml, Hq, Hkv, P, scale, window,     \
             num_splits);                                                                                \
         attention_decode_merge_kernel<D_><<<mgrid, 256, 0, stream>>>(part_acc, part_ml, dec_tokens,     \
-                                                                     (bf16_t*)out, Hq, num_splits);     \
+                                                                     (bf16_t*)out, Hq, num_splits, 0);  \
     } while (0)
     if (D == 128 && split_keys == 128) QE_DECODE_FUSED(128, 128);
     else if (D == 128) QE_DECODE_FUSED(128, 256);

@@ -38,7 +38,7 @@ __global__ __launch_bounds__(64 * F32_WAVES) void attention_f32_kernel(
     const float* __restrict__ q, float* __restrict__ out, const float* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ tok_seq,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tokens,
-    int Hq, int Hkv, int P, float scale, int window) {
+    int Hq, int Hkv, int P, float scale, int window, int keep_first, int sink) {
     constexpr int D = DB * 16;
     extern __shared__ float merge_lds[];                  // [F32_WAVES][DB * 4 + 2][64]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, n = lane & 15;
@@ -65,10 +65,18 @@ __global__ __launch_bounds__(64 * F32_WAVES) void attention_f32_kernel(
 #pragma unroll
     for (int db = 0; db < DB; ++db) acc[db] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    for (int kk = (lo / 16) * 16 + 16 * wave; kk <= p; kk += 16 * F32_WAVES) {
+    // The tiles of the walk: those of the kept first keys 0 .. kf - 1 that lie wholly before the window's
+    // first tile, then the tiles from the window's first on (which holds the rest of the kept keys, if
+    // any); tile number i of this list goes to wave i % F32_WAVES.
+    const int kf = keep_first < lo ? keep_first : lo;
+    const int tile_lo = lo / 16;
+    const int n_first = (kf + 15) / 16 < tile_lo ? (kf + 15) / 16 : tile_lo;
+    const int n_tiles = n_first + p / 16 - tile_lo + 1;
+    for (int ti = wave; ti < n_tiles; ti += F32_WAVES) {
+        const int kk = 16 * (ti < n_first ? ti : tile_lo + ti - n_first);
         // S^T: this lane brings the key row kk + n
         const int key_r = kk + n;
-        const bool row_ok = key_r >= lo && key_r <= p;
+        const bool row_ok = (key_r >= lo || key_r < kf) && key_r <= p;
         floatx4 s = {0.f, 0.f, 0.f, 0.f};
         {
             const float* krow = cache;
@@ -87,7 +95,7 @@ __global__ __launch_bounds__(64 * F32_WAVES) void attention_f32_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int key = kk + 4 * g + i;
-            ok[i] = key >= lo && key <= p;
+            ok[i] = (key >= lo || key < kf) && key <= p;
             s[i] = ok[i] ? s[i] * scale : -INFINITY;
             tmax = fmaxf(tmax, s[i]);
         }
@@ -141,10 +149,10 @@ __global__ __launch_bounds__(64 * F32_WAVES) void attention_f32_kernel(
     mine[(DB * 4 + 1) * 64] = l;
     __syncthreads();
     if (wave != 0) return;
-    float M = -INFINITY;
+    float M = sink ? 0.f : -INFINITY;                     // (the sink: one more entry of score 0 without a value)
 #pragma unroll
     for (int w = 0; w < F32_WAVES; ++w) M = fmaxf(M, merge_lds[((long)w * (DB * 4 + 2) + DB * 4) * 64 + lane]);
-    float wgt[F32_WAVES], lsum = 0.f;
+    float wgt[F32_WAVES], lsum = sink ? expf(-M) : 0.f;
 #pragma unroll
     for (int w = 0; w < F32_WAVES; ++w) {
         const float mw = merge_lds[((long)w * (DB * 4 + 2) + DB * 4) * 64 + lane];
@@ -175,7 +183,7 @@ bool qe_attention_f32_ok(int Hq, int Hkv, int D, int P) {
 
 int qe_attention_f32(const float* q, float* out, const float* cache, const int* positions, const int* tok_seq,
                      const int* block_table, int max_blocks, const int* tokens, int T, int Hq, int Hkv, int D,
-                     int P, float scale, int window, hipStream_t stream) {
+                     int P, float scale, int window, int keep_first, int sink, hipStream_t stream) {
     QE_REQUIRE(qe_attention_f32_ok(Hq, Hkv, D, P), "attention (32-bit): sizes not taken");
     const int groups16 = (Hq / Hkv + 15) / 16;
     QE_REQUIRE((long)Hkv * groups16 <= 65535, "attention (32-bit): too many heads");
@@ -193,7 +201,7 @@ int qe_attention_f32(const float* q, float* out, const float* cache, const int* 
             }                                                                                         \
         }                                                                                             \
         attention_f32_kernel<DB_><<<grid, 64 * F32_WAVES, lds, stream>>>(q, out, cache, positions, tok_seq, \
-                                                    block_table, max_blocks, tokens, Hq, Hkv, P, scale, window); \
+                                                    block_table, max_blocks, tokens, Hq, Hkv, P, scale, window, keep_first, sink); \
         break;                                                                                        \
     }
     switch (D / 16) {

@@ -5,10 +5,13 @@
 //
 // The query of token t at absolute position p = positions[t] of request
 // s = tok_seq[t] sees the keys at positions lo..p of that request, read through
-// block_table[s]; lo = 0, or p - window + 1 when a window is given.  Keys are
-// taken 64 at a time from lo upwards with an online softmax, so the order of the
-// sums depends on p and the window only: not on how the request's tokens were cut
-// into steps, nor on what else is in the batch.
+// block_table[s]; lo = 0, or p - window + 1 when a window is given.  With keep_first the
+// request's first keep_first keys are seen as well, wherever the window stands.  Keys are
+// taken 64 at a time, the kept first keys behind the window first, then from lo upwards, with
+// an online softmax, so the order of the sums depends on p, the window and keep_first only:
+// not on how the request's tokens were cut into steps, nor on what else is in the batch.
+// With sink the softmax has one more entry of score 0 that carries no value (a 1 in the
+// denominator): the running maximum starts at 0 with a sum of 1.
 //
 // cache of one layer: [page][2 (k, v)][Hkv][P * D]; a key tile is [P][D], a value tile is
 // stored transposed, [D][P] (the layout the MFMA kernels read without a shuffle).
@@ -21,7 +24,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const TA* __restrict__ q, TA* __restrict__ out, const TA* __restrict__ cache,
     const int* __restrict__ positions, const int* __restrict__ tok_seq,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tokens,
-    int Hq, int Hkv, int D, int P, float scale, int window) {
+    int Hq, int Hkv, int D, int P, float scale, int window, int keep_first, int sink) {
     extern __shared__ float smem[];
     float* qs = smem;            // D
     float* ps = smem + D;        // 64 probabilities of the current chunk
@@ -30,21 +33,24 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const int h = blockIdx.y;
     const int lane = threadIdx.x;
     const int kvh = h / (Hq / Hkv);
-    const int p = positions[t];
+    const int p_own = positions[t];
     const int* bt = block_table + (long)tok_seq[t] * max_blocks;
-    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int lo = (window > 0 && p_own - window + 1 > 0) ? p_own - window + 1 : 0;
     const long page_stride = 2L * Hkv * P * D;
 
     const TA* qrow = q + (t * Hq + h) * D;
     for (int d = lane; d < D; d += 64) qs[d] = Elem<TA>::load(qrow + d);
     __syncthreads();
 
-    float m = -INFINITY, l = 0.f;
+    float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
     float acc[ATTN_MAX_D / 64];
 #pragma unroll
     for (int i = 0; i < ATTN_MAX_D / 64; ++i) acc[i] = 0.f;
 
-    for (int j0 = lo; j0 <= p; j0 += 64) {
+    // two walks: the kept first keys that lie behind the window, 0 .. kf - 1, then lo .. p
+    const int kf = keep_first < lo ? keep_first : lo;
+    for (int walk = kf > 0 ? 0 : 1; walk < 2; ++walk)
+    for (int j0 = walk ? lo : 0, p = walk ? p_own : kf - 1; j0 <= p; j0 += 64) {
         const int j = j0 + lane;
         float sc = -INFINITY;
         long vo = 0;
@@ -91,7 +97,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
 bool qe_attention_f32_ok(int Hq, int Hkv, int D, int P);
 int qe_attention_f32(const float* q, float* out, const float* cache, const int* positions, const int* tok_seq,
                      const int* block_table, int max_blocks, const int* tokens, int T, int Hq, int Hkv, int D,
-                     int P, float scale, int window, hipStream_t stream);
+                     int P, float scale, int window, int keep_first, int sink, hipStream_t stream);
 
 // 32-bit attention goes to the kernel on the matrix units (attention_f32.hip) where it takes the
 // sizes, unless qe_use_matrix_f32(0) has switched that off.
@@ -99,11 +105,11 @@ extern int g_qe_matrix_f32;
 
 int qe_attention_generic(const void* q, void* out, const void* cache, const int* positions,
                          const int* tok_seq, const int* block_table, int max_blocks, const int* tokens,
-                         int T, int Hq, int Hkv, int D, int P, float scale, int window, int dt_a,
-                         hipStream_t stream) {
+                         int T, int Hq, int Hkv, int D, int P, float scale, int window, int keep_first, int sink,
+                         int dt_a, hipStream_t stream) {
     if (dt_a == QE_F32 && g_qe_matrix_f32 && qe_attention_f32_ok(Hq, Hkv, D, P))
         return qe_attention_f32((const float*)q, (float*)out, (const float*)cache, positions, tok_seq, block_table,
-                                max_blocks, tokens, T, Hq, Hkv, D, P, scale, window, stream);
+                                max_blocks, tokens, T, Hq, Hkv, D, P, scale, window, keep_first, sink, stream);
     QE_REQUIRE(D <= ATTN_MAX_D, "attention: head_dim=%d exceeds %d", D, ATTN_MAX_D);
     QE_REQUIRE(Hq <= 65535, "attention: too many heads");
     dim3 grid(T, Hq);
@@ -111,11 +117,11 @@ int qe_attention_generic(const void* q, void* out, const void* cache, const int*
     if (dt_a == QE_F32)
         attention_generic_kernel<float><<<grid, 64, shmem, stream>>>(
             (const float*)q, (float*)out, (const float*)cache, positions, tok_seq, block_table,
-            max_blocks, tokens, Hq, Hkv, D, P, scale, window);
+            max_blocks, tokens, Hq, Hkv, D, P, scale, window, keep_first, sink);
     else if (dt_a == QE_BF16)
         attention_generic_kernel<bf16_t><<<grid, 64, shmem, stream>>>(
             (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, positions, tok_seq, block_table,
-            max_blocks, tokens, Hq, Hkv, D, P, scale, window);
+            max_blocks, tokens, Hq, Hkv, D, P, scale, window, keep_first, sink);
     else
         QE_REQUIRE(false, "attention: unknown dtype %d", dt_a);
     QE_LAUNCH_CHECK();

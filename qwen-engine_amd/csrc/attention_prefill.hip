@@ -113,7 +113,7 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
     const int* __restrict__ tiles, const int* __restrict__ positions, const int* __restrict__ tok_seq,
     const int* __restrict__ block_table, int max_blocks,
     int Hq, int Hkv, int P, int log2P, float scale_log2, int window, int R, int seg_param, int keys_row,
-    float* __restrict__ part) {
+    float* __restrict__ part, int keep_first, int sink) {
     constexpr int KROW = D * 2 + 16;                 // bytes of a staged key row
     constexpr int KBYTES = 32 * KROW, VBYTES = 2 * D * VROW, BUF = KBYTES + VBYTES;
     constexpr int KP = 32 * (D / 8) / 256;           // 16-byte key pieces per thread (2 for D = 128)
@@ -145,6 +145,8 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
     const int p_block = positions[row_first];
     int kmin = (window > 0 && p_block - window + 1 > 0) ? p_block - window + 1 : 0;
     int kmax = positions[bt4[2 * last]] + bt4[2 * last + 1];
+    // the request's kept first keys that lie behind the block's window: [0, kfb) (never together with segments)
+    const int kfb = keep_first < kmin ? keep_first : kmin;
     // key segments: this block walks the keys of segment bseg only
     bool partial = false;
     const int seg_keys = segment_keys(seg_param, positions, keys_row);
@@ -227,7 +229,8 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
     const int page_bytes = (int)page_stride * 2;
 #define STAGE_LOAD(set_, kk_)                                                                       \
     {                                                                                               \
-        const bool first_ = (kk_) + 16 > kmin, second_ = (kk_) + 16 < kmax;                         \
+        const bool first_ = (kk_) + 16 > kmin || (kk_) < kfb;                                       \
+        const bool second_ = ((kk_) + 16 < kmax && (kk_) + 32 > kmin) || (kk_) + 16 < kfb;          \
         const int ka_ = first_ ? (kk_) : (kk_) + 16;                                                \
         const int kb_ = second_ ? (kk_) + 16 : (kk_);                                               \
         const __amdgpu_buffer_rsrc_t ra_ = __builtin_amdgcn_make_buffer_rsrc(                       \
@@ -250,7 +253,7 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
                 const int half = id / (2 * D), part = id & 1;                                       \
                 _Pragma("unroll") for (int e = 0; e < 8; ++e) {                                     \
                     const int key = (kk_) + 16 * half + 8 * part + e;                               \
-                    if (key < kmin || key >= kmax) vst[set_][i].e[e] = 0;                           \
+                    if ((key < kmin && key >= kfb) || key >= kmax) vst[set_][i].e[e] = 0;           \
                 }                                                                                   \
             }                                                                                       \
         }                                                                                           \
@@ -271,9 +274,12 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
     // The group's i-th tile holds the keys from kk0 + 32 (NG i + grp) on and uses register set and
     // shared buffer i % 2.  All groups make the same number of rounds (the barriers are the
     // block's); a round whose tile lies beyond the keys brings and computes nothing.
+    // The walk's tiles: those of the kept first keys that lie wholly before the window's first tile, then
+    // the tiles from the window's first on.
     const int kk0 = (kmin / 32) * 32;
-    const int rounds = ((kmax - kk0 + 31) / 32 + NG - 1) / NG;
-#define TILE_KEY(i_) (kk0 + 32 * (NG * (i_) + grp))
+    const int n_first = (kfb + 31) / 32 < kk0 / 32 ? (kfb + 31) / 32 : kk0 / 32;
+    const int rounds = (n_first + (kmax - kk0 + 31) / 32 + NG - 1) / NG;
+#define TILE_KEY(i_) (NG * (i_) + grp < n_first ? 32 * (NG * (i_) + grp) : kk0 + 32 * (NG * (i_) + grp - n_first))
     const int kk_first = TILE_KEY(0), kk_second = TILE_KEY(1);
     if (kk_first < kmax) {
         STAGE_LOAD(0, kk_first)
@@ -295,7 +301,7 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
         const int kk_1 = TILE_KEY(i + 1), kk_2 = TILE_KEY(i + 2);   // (values, not expressions in i: the macros have loops over i)
         STAGE_LOAD(buf, EXISTING(kk_2))                   // this set's tile went to shared memory a round ago
         __builtin_amdgcn_sched_barrier(0);                // keep the loads ahead of the computation
-        if (wave_on && kk < k_stop && kk + 32 > k_start && kk < kmax) {   // some row of the wave sees some key of the tile, and it is a tile of this block's keys
+        if (wave_on && kk < k_stop && (kk + 32 > k_start || kk < keep_first) && kk < kmax) {   // some row of the wave sees some key of the tile, and it is a tile of this block's keys
             const unsigned char* ks_ = smem + buf * BUF + r * KROW + g * 16;
             const unsigned char* vs_ = smem + buf * BUF + KBYTES + r * VROW + g * 16;
             // all key fragments are read before the first MFMA, all value fragments before the
@@ -321,14 +327,14 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
             // (the scores stay unscaled: the scale is positive, so it is applied to the maximum, and
             // to each score by the multiply-add that also subtracts the maximum)
             float tmax = -INFINITY;
-            if (kk >= all_lo && kk + 32 <= all_hi) {       // every column sees every key of the tile
+            if ((kk >= all_lo || kk + 32 <= keep_first) && kk + 32 <= all_hi) {   // every column sees every key of the tile
 #pragma unroll
                 for (int e = 0; e < 16; ++e) tmax = fmaxf(tmax, s[e]);
             } else {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const int key = kk + 8 * (e >> 2) + 4 * g + (e & 3);
-                    s[e] = (key >= lo && key < hi) ? s[e] : -INFINITY;
+                    s[e] = ((key >= lo || key < keep_first) && key < hi) ? s[e] : -INFINITY;
                     tmax = fmaxf(tmax, s[e]);
                 }
             }
@@ -416,6 +422,8 @@ __global__ __launch_bounds__(256 * NG, NG == 1 ? 2 : 1) void attention_prefill_k
         }
         return;
     }
+    // (sink: one more entry of score 0 that carries no value; m is the scaled reference of the weights)
+    if (sink) l += __builtin_amdgcn_exp2f(fminf(-m, 126.f));
     if (col_ok) store_columns<D>(out, acc, 1.f / l, row, head, Hq, g);
 }
 
@@ -559,7 +567,9 @@ int qe_attention_prefill(const void* q, void* out, const void* cache, const int*
                          const int* positions, const int* tok_seq, const int* block_table, int max_blocks,
                          int Hq, int Hkv, int D, int P, float scale, int window, int groups,
                          int seg_keys, int max_keys, int keys_row, void* workspace, size_t workspace_bytes,
-                         hipStream_t stream) {
+                         hipStream_t stream, int keep_first, int sink) {
+    QE_REQUIRE(seg_keys == 0 || (keep_first == 0 && !sink),
+               "prefill attention: kept first keys and a sink go with uncut walks only");
     QE_REQUIRE((D == 64 || D == 128) && P >= 16 && (P & (P - 1)) == 0 && Hq % Hkv == 0,
                "prefill attention: sizes not taken");
     int log2P = 0;
@@ -594,7 +604,7 @@ int qe_attention_prefill(const void* q, void* out, const void* cache, const int*
 #define QE_PREFILL(D_, NG_)                                                                         \
     attention_prefill_kernel<D_, NG_><<<grid, 256 * NG_, 0, stream>>>(                              \
         (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, tiles, positions, tok_seq, block_table, \
-        max_blocks, Hq, Hkv, P, log2P, scale_log2, window, R, seg_keys, keys_row, (float*)workspace)
+        max_blocks, Hq, Hkv, P, log2P, scale_log2, window, R, seg_keys, keys_row, (float*)workspace, keep_first, sink)
     if (D == 128) { if (groups == 2) QE_PREFILL(128, 2); else QE_PREFILL(128, 1); }
     else          { if (groups == 2) QE_PREFILL(64, 2); else QE_PREFILL(64, 1); }
 #undef QE_PREFILL

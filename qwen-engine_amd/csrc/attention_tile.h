@@ -78,10 +78,11 @@ struct AttnState {
 };
 
 // The tile's keys are kk .. kk + 15; this lane's column sees the keys in [lo, hi); [vlo, vhi) is
-// the range that any column of the wave sees (keys outside it may be unwritten memory).
+// the range that any column of the wave sees (keys outside it may be unwritten memory).  Keys below
+// kf are seen as well, by every column (a request's kept first keys, where a window is given).
 template <int D>
 __device__ __forceinline__ void attn_tile_step(AttnState<D>& st, const KVTile<D>& tile, const bf16x8 (&qreg)[D / 32],
-                                               float scale, int kk, int g, int lo, int hi, int vlo, int vhi) {
+                                               float scale, int kk, int g, int lo, int hi, int vlo, int vhi, int kf = 0) {
     floatx4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tile.k[c], qreg[c], s, 0, 0, 0);
@@ -90,7 +91,7 @@ __device__ __forceinline__ void attn_tile_step(AttnState<D>& st, const KVTile<D>
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int key = kk + g * 4 + j;
-        ok[j] = key >= lo && key < hi;
+        ok[j] = (key >= lo && key < hi) || key < kf;
         s[j] = ok[j] ? s[j] * scale : -INFINITY;
         tmax = fmaxf(tmax, s[j]);
     }
@@ -115,7 +116,7 @@ __device__ __forceinline__ void attn_tile_step(AttnState<D>& st, const KVTile<D>
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int key = kk + g * 4 + j;
-        vmask[j] = (short)((key >= vlo && key < vhi) ? -1 : 0);
+        vmask[j] = (short)(((key >= vlo && key < vhi) || key < kf) ? -1 : 0);
     }
 #pragma unroll
     for (int db = 0; db < D / 16; ++db) {

@@ -59,6 +59,8 @@ struct QkvTail {
     // With SILU: act_limit > 0 makes the activation min(g, limit) sigmoid(act_slope g) (clamp(u, -limit, limit) + 1)
     // instead of silu(g) u.
     float act_limit, act_slope;
+    // Without SILU: the result is relu(.)^2 instead of the product itself.
+    int relu_sq;
 };
 
 // BIG (256 x 256 by four waves, one wave a SIMD, a wave's part 128 x 128): the accumulators fill the
@@ -523,6 +525,7 @@ __global__ __launch_bounds__(64 * NW, MINB) void gemm_mfma_kernel(
                         v[r] = gt * __builtin_amdgcn_rcpf(1.f + __expf(-slope * gt)) * up;   // rcp: within 1 ulp
                     } else {
                         v[r] = acc[i][j][4 * bq + r];
+                        if (tail.relu_sq) { const float z = fmaxf(v[r], 0.f); v[r] = z * z; }
                     }
                 }
                 if (!SILU && bias && blockIdx.y == 0) {                       // (a column beyond the output is never stored: any bias does)
@@ -596,7 +599,7 @@ static int launch_mfma(const void* x, const void* w, const float* bias, void* ou
 // Rows grouped by expert against one matrix per expert (see QkvTail): tiles of 128 x 128.
 template <typename TO, bool SILU>
 static int launch_grouped(const void* x, const void* w, void* out, const int* tiles, const int* n_tiles,
-                          int max_tiles, int N, int K, float limit, float slope, hipStream_t stream) {
+                          int max_tiles, int N, int K, float limit, float slope, hipStream_t stream, int relu_sq = 0) {
     constexpr int BM = 128, BN = 128, BK = 64, NW = 4;
     const int tiles_n = qe_cdiv(N, BN);
     const long blocks = (long)max_tiles * tiles_n;
@@ -613,6 +616,7 @@ static int launch_grouped(const void* x, const void* w, void* out, const int* ti
     tail.n_tiles = n_tiles;
     tail.act_limit = limit;
     tail.act_slope = slope;
+    tail.relu_sq = relu_sq;
     gemm_mfma_kernel<TO, BM, BN, BK, NW, 2, SILU, false><<<dim3((unsigned)blocks, 1), 64 * NW, shmem, stream>>>(
         (const bf16_t*)x, (const bf16_t*)w, nullptr, (TO*)out, 0, N, K, max_tiles, tiles_n, K, 0, 0, 0, tail);
     QE_LAUNCH_CHECK();
@@ -625,8 +629,12 @@ extern "C" int qe_gemm_mfma_grouped(const void* x, const void* w, void* out, con
                                     int max_tiles, int N, int K, int silu, float limit, float slope, int dt_o,
                                     hipStream_t stream) {
     QE_REQUIRE(K % 8 == 0 && K >= 64, "mfma gemm (grouped): K=%d", K);
-    QE_REQUIRE(!silu || N % 64 == 0, "mfma gemm (grouped): gate|up rows in blocks of 32");
+    QE_REQUIRE(silu != 1 || N % 64 == 0, "mfma gemm (grouped): gate|up rows in blocks of 32");
     if (max_tiles == 0) return 0;
+    if (silu == 2) {       // one matrix an expert, the result relu(.)^2
+        QE_REQUIRE(dt_o == QE_BF16, "mfma gemm (grouped): the activation is stored in bfloat16");
+        return launch_grouped<bf16_t, false>(x, w, out, tiles, n_tiles, max_tiles, N, K, 0.f, 1.f, stream, 1);
+    }
     if (silu) {
         QE_REQUIRE(dt_o == QE_BF16, "mfma gemm (grouped): the activation is stored in bfloat16");
         return launch_grouped<bf16_t, true>(x, w, out, tiles, n_tiles, max_tiles, N, K, limit, slope, stream);

@@ -6,6 +6,11 @@
 //                  of neighbours; a group's score is its largest; only the experts of the ``keep`` best
 //                  groups can be chosen; of those the ``top`` largest are, weighted by their scores as
 //                  they are.  On ties the lower index wins.  ids [T, top], weights [T, top].
+//   qe_moe_route_biased  scores = softmax(logits) over all experts (32-bit); the ``top`` largest of
+//                  score + correction are chosen (on ties the lower index), weighted by their scores
+//                  without the correction, divided by the chosen scores' sum (+ 1e-20), times ``scale``.
+//   qe_moe_identity  the experts from E_real on are the identity: a pair that chose one contributes its
+//                  token's row itself; they get no tiles from qe_moe_sort (tile_experts).
 //   qe_moe_sort    perm [T * top]: the pairs (as index t * top + j) ordered by expert; tiles
 //                  [max_tiles, 3] = (expert, first sorted row, rows <= tile_rows) and their number.
 //   qe_moe_gather  xs[i] = x[perm[i] / top]: the pairs' rows side by side, for a product that wants its rows
@@ -18,6 +23,7 @@
 //                    second product (weighted): a's sorted row against W_e [N, K], times the pair's
 //                      weight, to parts[j][t] (32-bit): the norm that follows adds a token's ``top``
 //                      parts in the order of j.
+//                    dual == 2: one matrix W_e [F, K] and a = relu(W_e x)^2 instead.
 //                  Any sizes, every multiply-add in IEEE 32-bit.
 #include "common.h"
 
@@ -100,8 +106,104 @@ extern "C" int qe_moe_route(const float* logits, int* ids, float* weights, int T
     return 0;
 }
 
-// One block.  n = T * top pairs.
-__global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ ids, int n, int E, int tile_rows,
+
+// One wave per token: softmax over all E experts, choice by score + correction, weights from the scores alone.
+__global__ __launch_bounds__(64) void moe_route_biased_kernel(const float* __restrict__ logits, const float* __restrict__ correction,
+                                                              int* __restrict__ ids, float* __restrict__ weights, int E, int top,
+                                                              float scale) {
+    extern __shared__ float sc[];          // E scores, E choice scores, top chosen scores
+    float* ch = sc + E;
+    float* picked = ch + E;
+    const long t = blockIdx.x;
+    const int lane = threadIdx.x;
+    const float* z = logits + t * E;
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) {
+        const float ex = expf(z[e] - mx);
+        sc[e] = ex;
+        sum += ex;
+    }
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += 64) {
+        float v = sc[e] / sum;
+        if (!(v == v)) v = 0.f;            // (a row of garbage still gets experts inside the table)
+        sc[e] = v;
+        float c = v + correction[e];
+        if (!(c == c)) c = 0.f;
+        ch[e] = c;
+    }
+    __syncthreads();
+    for (int r = 0; r < top; ++r) {
+        float bv = -INFINITY;
+        int bi = -1;
+        for (int e = lane; e < E; e += 64)
+            if (ch[e] > bv) { bv = ch[e]; bi = e; }
+        wave_argmax(bv, bi);
+        if (lane == 0) {
+            ids[t * top + r] = bi >= 0 ? bi : 0;
+            picked[r] = bi >= 0 ? sc[bi] : 0.f;
+            if (bi >= 0) ch[bi] = -INFINITY;
+        }
+        __syncthreads();
+    }
+    if (lane == 0) {
+        float tot = 0.f;
+        for (int r = 0; r < top; ++r) tot += picked[r];
+        for (int r = 0; r < top; ++r) weights[t * top + r] = picked[r] / (tot + 1e-20f) * scale;
+    }
+}
+
+extern "C" int qe_moe_route_biased(const float* logits, const float* correction, int* ids, float* weights, int T, int E,
+                                   int top, float scale, hipStream_t stream) {
+    QE_REQUIRE(T >= 0 && E > 0 && top >= 1 && top <= E, "moe_route_biased: top %d of %d experts", top, E);
+    QE_REQUIRE((2 * E + top) * sizeof(float) <= 60000, "moe_route_biased: too many experts");
+    if (T == 0) return 0;
+    moe_route_biased_kernel<<<T, 64, (2 * E + top) * sizeof(float), stream>>>(logits, correction, ids, weights, E, top, scale);
+    QE_LAUNCH_CHECK();
+    return 0;
+}
+
+// One block per (token, choice) pair that chose an identity expert (id >= E_real): its part of the output is the
+// token's row itself.  parts != null: parts[j][t] = weight * x[t] (32-bit); else y[inv[pair]] = x[t] (32-bit), for a
+// caller that weighs and adds the sorted rows afterwards.
+template <typename TA>
+__global__ void moe_identity_kernel(const TA* __restrict__ x, const int* __restrict__ ids, const float* __restrict__ weights,
+                                    const int* __restrict__ inv, float* __restrict__ parts, float* __restrict__ y,
+                                    int T, int top, int H, int E_real) {
+    const long pair = blockIdx.x;
+    if (ids[pair] < E_real) return;
+    const long t = pair / top;
+    const int j = pair % top;
+    const TA* src = x + t * H;
+    if (parts) {
+        const float wgt = weights[pair];
+        float* dst = parts + ((long)j * T + t) * H;
+        for (int c = threadIdx.x; c < H; c += blockDim.x) dst[c] = wgt * Elem<TA>::load(src + c);
+    } else {
+        float* dst = y + (long)inv[pair] * H;
+        for (int c = threadIdx.x; c < H; c += blockDim.x) dst[c] = Elem<TA>::load(src + c);
+    }
+}
+
+extern "C" int qe_moe_identity(const void* x, const int* ids, const float* weights, const int* inv, float* parts, float* y,
+                               int T, int top, int H, int E_real, int dt_a, hipStream_t stream) {
+    QE_REQUIRE(T >= 0 && top > 0 && H > 0 && E_real >= 0, "moe_identity: bad sizes");
+    QE_REQUIRE((parts != nullptr) != (y != nullptr), "moe_identity: parts or sorted rows, one of them");
+    QE_REQUIRE(parts || inv, "moe_identity: sorted rows need the pairs' places");
+    if (T == 0) return 0;
+    if (dt_a == QE_BF16) moe_identity_kernel<bf16_t><<<T * top, 256, 0, stream>>>((const bf16_t*)x, ids, weights, inv, parts, y, T, top, H, E_real);
+    else if (dt_a == QE_F32) moe_identity_kernel<float><<<T * top, 256, 0, stream>>>((const float*)x, ids, weights, inv, parts, y, T, top, H, E_real);
+    else QE_REQUIRE(false, "moe_identity: unknown type %d", dt_a);
+    QE_LAUNCH_CHECK();
+    return 0;
+}
+
+// One block.  n = T * top pairs.  Only the first tile_experts experts get tiles (the others' pairs still get
+// their places in perm, behind them).
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ ids, int n, int E, int tile_experts, int tile_rows,
                                                         int* __restrict__ perm, int* __restrict__ inv,
                                                         int* __restrict__ tiles, int* __restrict__ n_tiles) {
     extern __shared__ int sm[];
@@ -116,17 +218,17 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ 
         int off = 0, tb = 0;
         for (int j = 0; j < e; ++j) {
             off += counts[j];
-            tb += (counts[j] + tile_rows - 1) / tile_rows;
+            if (j < tile_experts) tb += (counts[j] + tile_rows - 1) / tile_rows;
         }
         cursor[e] = off;
         const int c = counts[e];
-        const int mine = (c + tile_rows - 1) / tile_rows;
+        const int mine = e < tile_experts ? (c + tile_rows - 1) / tile_rows : 0;
         for (int k = 0; k < mine; ++k) {
             tiles[3 * (tb + k)] = e;
             tiles[3 * (tb + k) + 1] = off + k * tile_rows;
             tiles[3 * (tb + k) + 2] = c - k * tile_rows < tile_rows ? c - k * tile_rows : tile_rows;
         }
-        if (e == E - 1) n_tiles[0] = tb + mine;
+        if (e == tile_experts - 1) n_tiles[0] = tb + mine;
     }
     __syncthreads();
     for (int i = tid; i < n; i += blockDim.x) {
@@ -137,12 +239,12 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ 
 }
 
 // inv (may be null): the sorted row of every pair, perm's inverse
-extern "C" int qe_moe_sort(const int* ids, int n, int E, int tile_rows, int* perm, int* inv, int* tiles, int* n_tiles,
-                           int max_tiles, hipStream_t stream) {
-    QE_REQUIRE(n >= 0 && E > 0 && tile_rows > 0, "moe_sort: bad sizes");
-    QE_REQUIRE(max_tiles >= (n + tile_rows - 1) / tile_rows + (E < n ? E : n), "moe_sort: %d tiles may not be enough", max_tiles);
+extern "C" int qe_moe_sort(const int* ids, int n, int E, int tile_experts, int tile_rows, int* perm, int* inv, int* tiles,
+                           int* n_tiles, int max_tiles, hipStream_t stream) {
+    QE_REQUIRE(n >= 0 && E > 0 && tile_rows > 0 && tile_experts >= 1 && tile_experts <= E, "moe_sort: bad sizes");
+    QE_REQUIRE(max_tiles >= (n + tile_rows - 1) / tile_rows + (tile_experts < n ? tile_experts : n), "moe_sort: %d tiles may not be enough", max_tiles);
     QE_REQUIRE(2 * E * sizeof(int) <= 60000, "moe_sort: too many experts");
-    moe_sort_kernel<<<1, 1024, 2 * E * sizeof(int), stream>>>(ids, n, E, tile_rows, perm, inv, tiles, n_tiles);
+    moe_sort_kernel<<<1, 1024, 2 * E * sizeof(int), stream>>>(ids, n, E, tile_experts, tile_rows, perm, inv, tiles, n_tiles);
     QE_LAUNCH_CHECK();
     return 0;
 }
@@ -150,11 +252,12 @@ extern "C" int qe_moe_sort(const int* ids, int n, int E, int tile_rows, int* per
 #define MT 64
 #define MK 16
 
-template <typename TA, typename TW, bool DUAL>
+template <typename TA, typename TW, int MODE>      // 0: second product, weighted; 1: gate and up; 2: one matrix, squared relu
 __global__ __launch_bounds__(256) void moe_gemm_kernel(
     const TA* __restrict__ x, const int* __restrict__ perm, int top, const TW* __restrict__ w, void* __restrict__ out_,
     const float* __restrict__ weights, const int* __restrict__ tiles, const int* __restrict__ n_tiles, int T, int N,
     int K, float limit, float slope, int interleaved) {
+    constexpr bool DUAL = MODE == 1, FIRST = MODE != 0;
     if ((int)blockIdx.y >= n_tiles[0]) return;
     __shared__ float xs[MK][MT + 4];
     __shared__ float ws[MK][MT + 4];
@@ -163,7 +266,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
     const int tid = threadIdx.x;
     const int e = tiles[3 * blockIdx.y], r0 = tiles[3 * blockIdx.y + 1], rows = tiles[3 * blockIdx.y + 2];
     const int n0 = blockIdx.x * MT;
-    if (tid < MT) src[tid] = tid < rows ? (DUAL ? perm[r0 + tid] / top : r0 + tid) : -1;
+    if (tid < MT) src[tid] = tid < rows ? (FIRST ? perm[r0 + tid] / top : r0 + tid) : -1;
     __syncthreads();
     const int lr = tid >> 2;
     const int lk = (tid & 3) * 4;
@@ -215,7 +318,16 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
     for (int i = 0; i < 4; ++i) {
         const int m = ty * 4 + i;
         if (m >= rows) continue;
-        if (DUAL) {
+        if (MODE == 2) {
+            TA* o = (TA*)out_ + (long)(r0 + m) * N;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int n = n0 + tx * 4 + j;
+                if (n >= N) continue;
+                const float z = fmaxf(acc[i][j], 0.f);
+                Elem<TA>::store(o + n, z * z);
+            }
+        } else if (DUAL) {
             TA* o = (TA*)out_ + (long)(r0 + m) * N;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -240,6 +352,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(
 
 // dual != 0: x [T, K] rows of the pairs' tokens, w [E, 2 N, K] (gate rows then up rows, or, interleaved, in
 // alternating blocks of 32), out [T * top, N] in x's type at the sorted rows.
+// dual == 2: the same rows, w [E, N, K], out relu(.)^2 at the sorted rows.
 // dual == 0: x [T * top, K] sorted rows, w [E, N, K], out float [top, T, N].
 extern "C" int qe_moe_gemm(const void* x, const int* perm, int top, const void* w, void* out, const float* weights,
                            const int* tiles, const int* n_tiles, int max_tiles, int T, int N, int K, float limit,
@@ -249,8 +362,9 @@ extern "C" int qe_moe_gemm(const void* x, const int* perm, int top, const void* 
     dim3 grid(qe_cdiv(N, MT), max_tiles);
 #define QE_MG(TA_, TW_)                                                                                              \
     do {                                                                                                             \
-        if (dual) moe_gemm_kernel<TA_, TW_, true><<<grid, 256, 0, stream>>>((const TA_*)x, perm, top, (const TW_*)w, out, weights, tiles, n_tiles, T, N, K, limit, slope, interleaved); \
-        else moe_gemm_kernel<TA_, TW_, false><<<grid, 256, 0, stream>>>((const TA_*)x, perm, top, (const TW_*)w, out, weights, tiles, n_tiles, T, N, K, limit, slope, interleaved);     \
+        if (dual == 2) moe_gemm_kernel<TA_, TW_, 2><<<grid, 256, 0, stream>>>((const TA_*)x, perm, top, (const TW_*)w, out, weights, tiles, n_tiles, T, N, K, limit, slope, interleaved); \
+        else if (dual) moe_gemm_kernel<TA_, TW_, 1><<<grid, 256, 0, stream>>>((const TA_*)x, perm, top, (const TW_*)w, out, weights, tiles, n_tiles, T, N, K, limit, slope, interleaved); \
+        else moe_gemm_kernel<TA_, TW_, 0><<<grid, 256, 0, stream>>>((const TA_*)x, perm, top, (const TW_*)w, out, weights, tiles, n_tiles, T, N, K, limit, slope, interleaved);     \
     } while (0)
     if (dt_a == QE_F32 && dt_w == QE_F32) QE_MG(float, float);
     else if (dt_a == QE_BF16 && dt_w == QE_BF16) QE_MG(bf16_t, bf16_t);

@@ -13,11 +13,12 @@
 // KSPLIT (with MT == 1, few rows): the block's four waves take the same 16 features and a quarter of K each
 // (steps of 32 in turn), and wave 0 adds the four parts in the order of the waves: four times the blocks, for
 // a product that is bound by streaming the weights of the few experts that a handful of tokens choose.
-template <int MT, bool DUAL, bool KSPLIT = false>
+template <int MT, int MODE, bool KSPLIT = false>     // MODE 0: second product, weighted; 1: gate and up; 2: one matrix, squared relu
 __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(
     const bf16_t* __restrict__ x, const int* __restrict__ perm, int top, const bf16_t* __restrict__ w,
     void* __restrict__ out_, const float* __restrict__ weights, const int* __restrict__ tiles,
     const int* __restrict__ n_tiles, int T, int N, int K, float limit, float slope, int interleaved) {
+    constexpr bool DUAL = MODE == 1, FIRST = MODE != 0;
     if ((int)blockIdx.y >= n_tiles[0]) return;
     const int e = tiles[3 * blockIdx.y], r0 = tiles[3 * blockIdx.y + 1], rows = tiles[3 * blockIdx.y + 2];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, g = lane >> 4, nn = lane & 15;
@@ -33,7 +34,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(
     for (int i = 0; i < MT; ++i) {
         const int m = i * 16 + nn;
         const int mr = m < rows ? m : 0;
-        const long src = DUAL ? perm[r0 + mr] / top : r0 + mr;
+        const long src = FIRST ? perm[r0 + mr] / top : r0 + mr;
         xr[i] = x + src * K + g * 8;
     }
     floatx4 ag[MT], au[MT];
@@ -73,7 +74,15 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(
     for (int i = 0; i < MT; ++i) {
         const int m = i * 16 + nn;
         if (m >= rows) continue;
-        if (DUAL) {
+        if (MODE == 2) {
+            bf16_t* o = (bf16_t*)out_ + (long)(r0 + m) * N + n0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (n0 + j >= N) break;
+                const float z = fmaxf(ag[i][j], 0.f);
+                Elem<bf16_t>::store(o + j, z * z);
+            }
+        } else if (DUAL) {
             bf16_t* o = (bf16_t*)out_ + (long)(r0 + m) * N + n0;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -95,7 +104,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(
 
 extern "C" int qe_moe_gemm_mfma_supported(int K) { return K > 0 && K % 8 == 0; }
 
-// As qe_moe_gemm (moe.hip), bfloat16 only; the tiles were cut with ``tile_rows`` rows (16 or 64).
+// As qe_moe_gemm (moe.hip), bfloat16 only (dual == 2: one matrix and a squared relu); the tiles were cut with ``tile_rows`` rows (16 or 64).
 extern "C" int qe_moe_gemm_mfma(const void* x, const int* perm, int top, const void* w, void* out, const float* weights,
                                 const int* tiles, const int* n_tiles, int max_tiles, int tile_rows, int T, int N, int K,
                                 float limit, float slope, int dual, int interleaved, hipStream_t stream) {
@@ -107,9 +116,9 @@ extern "C" int qe_moe_gemm_mfma(const void* x, const int* perm, int top, const v
     const bool ksplit = tile_rows == 16 && max_tiles <= 64 && K >= 256;
     dim3 grid(qe_cdiv(N, ksplit ? 16 : 64), max_tiles);
 #define QE_MM(MT_, DUAL_, KS_) moe_gemm_mfma_kernel<MT_, DUAL_, KS_><<<grid, 256, 0, stream>>>((const bf16_t*)x, perm, top, (const bf16_t*)w, out, weights, tiles, n_tiles, T, N, K, limit, slope, interleaved)
-    if (ksplit) { if (dual) QE_MM(1, true, true); else QE_MM(1, false, true); }
-    else if (tile_rows == 16) { if (dual) QE_MM(1, true, false); else QE_MM(1, false, false); }
-    else { if (dual) QE_MM(4, true, false); else QE_MM(4, false, false); }
+    if (ksplit) { if (dual == 2) QE_MM(1, 2, true); else if (dual) QE_MM(1, 1, true); else QE_MM(1, 0, true); }
+    else if (tile_rows == 16) { if (dual == 2) QE_MM(1, 2, false); else if (dual) QE_MM(1, 1, false); else QE_MM(1, 0, false); }
+    else { if (dual == 2) QE_MM(4, 2, false); else if (dual) QE_MM(4, 1, false); else QE_MM(4, 0, false); }
 #undef QE_MM
     QE_LAUNCH_CHECK();
     return 0;

@@ -294,7 +294,8 @@ class ModelRunner:
                 first_key = 0 if grp.window is None else max(0, s.kv_before - grp.window + 1)
                 last_key = s.kv_before + s.q_len - 1
                 table = rc.tables[g]
-                for i in range(first_key // P, last_key // P + 1):
+                kept = range(0, min(self.cache.kept_first_pages(g), last_key // P + 1))
+                for i in [*kept, *range(first_key // P, last_key // P + 1)]:
                     if i >= len(table) or table[i] < 0:
                         raise RuntimeError(f"request {s.req_id!r} holds no page for position {i * P} of group {g}, "
                                            f"which its tokens at {s.kv_before}..{last_key} can see")

@@ -135,7 +135,8 @@ class Scheduler:
         P = self.cache.page_size
         for g, pool in enumerate(self.cache.pools):
             w = self.cache.groups[g].window
-            span = total_len if w is None else min(total_len, w + self.prefill_chunk + P)
+            span = total_len if w is None else min(total_len, w + self.prefill_chunk + P +
+                                                   self.cache.kept_first_pages(g) * P)
             if (span + P - 1) // P > pool.num_pages:
                 return False
         return True

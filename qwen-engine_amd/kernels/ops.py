@@ -59,7 +59,7 @@ def load_library():
         "qe_attention_decode_supported": [i32, i32, i32, i32, i32],
         "qe_attention_prefill_supported": [i32, i32, i32, i32, i32],
         "qe_attention_prefill_rows": [i32, i32],
-        "qe_attention_prefill_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, i32,
+        "qe_attention_prefill_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, i32, i32, i32,
                                      i32, vp, i64, vp],
         "qe_attention_prefill_plan_segments": [i32, i32, i32],
         "qe_attention_prefill_tiles_run": [vp, i32, i32, vp, i32, vp],
@@ -67,7 +67,7 @@ def load_library():
         "qe_attention_prefill_plan": [i32, i32, i32, i32],
         "qe_attention_prefill_plan_uncut_keys": [],
         "qe_attention_prefill_workspace_bytes": [i32, i32, i32, i32, i32, i32],
-        "qe_attention_decode_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, vp, i32, i32, i32, i32, f32, i32, i32, i32, vp, i64, vp],
+        "qe_attention_decode_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, vp, i32, i32, i32, i32, f32, i32, i32, i32, i32, i32, vp, i64, vp],
         "qe_attention_decode_fused_run": [vp, vp, vp, vp, i32, vp, vp, vp, i32, vp, vp, vp, vp, f32, vp,
                                           i32, i32, i32, i32, f32, i32, i32, i32, vp, i64, vp],
         "qe_qk_rope_store": [vp, vp, vp, vp, f32, vp, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp],
@@ -75,7 +75,11 @@ def load_library():
         "qe_qk_rope_store_parts_supported": [i32, i32],
         "qe_gemm_partial_preferred": [i32, i32, i32, i32, i32],
         "qe_gemm_branch_splits": [i32, i32, i32, i32, i32],
-        "qe_attention": [vp, vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp],
+        "qe_attention": [vp, vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, i32, vp],
+        "qe_qkv_conv_rope_store": [vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, vp],
+        "qe_scale_f32": [vp, i64, f32, vp],
+        "qe_moe_route_biased": [vp, vp, vp, vp, i32, i32, i32, f32, vp],
+        "qe_moe_identity": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp],
         "qe_argmax": [vp, vp, i32, i32, vp, i64, vp],
         "qe_argmax_static": [vp, vp, i32, i32, vp],
         "qe_sample": [vp, vp, vp, vp, i32, i32, vp],
@@ -91,7 +95,7 @@ def load_library():
         "qe_gemm_heads_mfma_supported": [i32, i64, i64],
         "qe_gemm_heads_mfma": [vp, i64, i64, vp, vp, i64, i64, vp, i32, i32, i32, i32, vp],
         "qe_moe_route": [vp, vp, vp, i32, i32, i32, i32, i32, vp],
-        "qe_moe_sort": [vp, i32, i32, i32, vp, vp, vp, vp, i32, vp],
+        "qe_moe_sort": [vp, i32, i32, i32, i32, vp, vp, vp, vp, i32, vp],
         "qe_moe_gemm": [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, f32, i32, i32, i32, i32, vp],
         "qe_moe_gather": [vp, vp, i32, vp, i32, i32, i32, vp],
         "qe_moe_combine": [vp, vp, vp, vp, i32, i32, i32, vp],
@@ -601,11 +605,15 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
               other_tokens: Optional[torch.Tensor] = None,
               other_tiles: Optional[torch.Tensor] = None, prefill_groups: int = 0,
               max_other_keys: int = 0, prefill_segment_keys: int = -1,
-              other_keys_row: Optional[int] = None, shared_keys: Optional[torch.Tensor] = None) -> torch.Tensor:
+              other_keys_row: Optional[int] = None, shared_keys: Optional[torch.Tensor] = None,
+              keep_first: int = 0, sink: bool = False) -> torch.Tensor:
     """q [T, Hq, D]; cache [pages, 2, Hkv, P, D] (key tiles [P][D], value tiles transposed [D][P]);
     positions, tok_seq int32 [T]; block_table int32 [B, max_blocks].  Token t sees the keys at
     positions max(0, p - window + 1) .. p of request tok_seq[t] (window 0: all).  The caller
-    guarantees that those positions have pages in the table.
+    guarantees that those positions have pages in the table.  With ``keep_first`` the request's first
+    keep_first keys are seen as well, wherever the window stands; with ``sink`` the softmax has a 1 added
+    to its denominator (one more entry of score 0 that carries no value).  Both go with uncut walks of the
+    prefill kernel only (no segments of keys).
 
     dec_tokens (int32 rows of q that are the single new token of their request, the largest of
     their positions being max_dec_position) go to the decode kernel where it takes the sizes;
@@ -638,12 +646,18 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
     max_blocks = block_table.shape[1]
     if shared_keys is not None:
         _need(shared_keys, "shared_keys", torch.int32, (block_table.shape[0],), dev)
+    keep_first, sink = int(keep_first) if window else 0, int(bool(sink))
+    if keep_first < 0:
+        raise KernelError("attention: negative keep_first")
+    if keep_first or sink:
+        prefill_segment_keys = 0
 
     def generic(tokens):
         n = T if tokens is None else tokens.shape[0]
         _check(lib.qe_attention(q.data_ptr(), out.data_ptr(), cache.data_ptr(), positions.data_ptr(),
                                 tok_seq.data_ptr(), block_table.data_ptr(), max_blocks, _ptr(tokens), n,
-                                Hq, Hkv, D, P, float(scale), int(window), _DT[q.dtype], _stream()), "attention")
+                                Hq, Hkv, D, P, float(scale), int(window), keep_first, sink, _DT[q.dtype], _stream()),
+               "attention")
 
     if dec_tokens is None and other_tokens is None:
         generic(None)
@@ -658,7 +672,7 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
                                                dec_tokens.data_ptr(), n_dec, positions.data_ptr(),
                                                tok_seq.data_ptr(), block_table.data_ptr(), max_blocks,
                                                _ptr(shared_keys), Hq, Hkv,
-                                               D, P, float(scale), int(window), int(max_dec_position),
+                                               D, P, float(scale), int(window), keep_first, sink, int(max_dec_position),
                                                DECODE_SPLIT_KEYS, ws.data_ptr(), nbytes, _stream()),
                    "attention (decode)")
         else:
@@ -691,7 +705,7 @@ def attention(q: torch.Tensor, cache: torch.Tensor, positions: torch.Tensor, tok
             _check(lib.qe_attention_prefill_run(q.data_ptr(), out.data_ptr(), cache.data_ptr(),
                                                 other_tiles.data_ptr(), n_tiles,
                                                 positions.data_ptr(), tok_seq.data_ptr(), block_table.data_ptr(),
-                                                max_blocks, Hq, Hkv, D, P, float(scale), int(window),
+                                                max_blocks, Hq, Hkv, D, P, float(scale), int(window), keep_first, sink,
                                                 int(prefill_groups), seg, max_keys, keys_row, _ptr(ws), nbytes,
                                                 _stream()),
                    "attention (prefill)")
@@ -1019,14 +1033,80 @@ def moe_route(logits: torch.Tensor, groups: int, keep: int, top: int):
     return ids, weights
 
 
+def moe_route_biased(logits: torch.Tensor, correction: torch.Tensor, top: int, scale: float):
+    """logits float32 [T, E], correction float32 [E] -> (ids int32 [T, top], weights float32 [T, top]): softmax
+    over all experts; the ``top`` largest of score + correction are chosen (the lower index on ties); their
+    weights are their scores without the correction, divided by the chosen scores' sum (+ 1e-20), times scale."""
+    lib = load_library()
+    _need(logits, "logits", torch.float32, (None, None))
+    T, E = logits.shape
+    _need(correction, "correction", torch.float32, (E,), logits.device)
+    ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    _check(lib.qe_moe_route_biased(logits.data_ptr(), correction.data_ptr(), ids.data_ptr(), weights.data_ptr(), T, E,
+                                   int(top), float(scale), _stream()), "moe_route_biased")
+    return ids, weights
+
+
+def scale_(x: torch.Tensor, s: float) -> None:
+    """x *= s on a 32-bit tensor."""
+    lib = load_library()
+    _need(x, "x", torch.float32)
+    _check(lib.qe_scale_f32(x.data_ptr(), x.numel(), float(s), _stream()), "scale")
+
+
+def qkv_conv_rope_store(qkv: torch.Tensor, conv_w: torch.Tensor, state: Optional[torch.Tensor], tok_seq: torch.Tensor,
+                        positions: torch.Tensor, inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor],
+                        cache: torch.Tensor, num_heads: int, num_kv_heads: int, k_dim: int, v_dim: int,
+                        single_rows: bool = False) -> torch.Tensor:
+    """What stands between a q|k|v projection and the attention where q, k and v each pass a short causal
+    convolution over time and q and k are then rotated on their first numbers.  qkv [T, Hq Dk + Hkv Dk + Hkv Dv];
+    conv_w float32 [that many, taps]; state float32 [slots, taps - 1, that many] (row tok_seq[t]: the request's last
+    projected rows; None for one tap), brought up to date; inv_freq float32 [rotated numbers / 2] or None.
+    cache [pages, 2, Hkv, P, Dc] with Dc >= Dk, Dv: keys and values go to slots[t] (negative or no slots:
+    nowhere), zeros beyond a head's own numbers.  Returns q [T, Hq, Dc], padded likewise.  The rows of a request
+    are consecutive; ``single_rows``: no two rows belong to the same request (one launch)."""
+    lib = load_library()
+    _need(qkv, "qkv", _ACT, (None, None))
+    T, C = qkv.shape
+    dev = qkv.device
+    Hq, Hkv, Dk, Dv = int(num_heads), int(num_kv_heads), int(k_dim), int(v_dim)
+    if C != Hq * Dk + Hkv * (Dk + Dv):
+        raise KernelError(f"qkv_conv_rope_store: rows of {C} are not {Hq} x {Dk} + {Hkv} x ({Dk} + {Dv})")
+    _need(conv_w, "conv_w", torch.float32, (C, None), dev)
+    taps = conv_w.shape[1]
+    if taps > 1:
+        if state is None:
+            raise KernelError("qkv_conv_rope_store: no state")
+        _need(state, "state", torch.float32, (None, taps - 1, C), dev)
+    _need(tok_seq, "tok_seq", torch.int32, (T,), dev)
+    _need(positions, "positions", torch.int32, (T,), dev)
+    rot = 0
+    if inv_freq is not None:
+        _need(inv_freq, "inv_freq", torch.float32, (None,), dev)
+        rot = 2 * inv_freq.shape[0]
+    _need(cache, "cache", qkv.dtype, (None, 2, Hkv, None, None), dev)
+    P, Dc = cache.shape[3], cache.shape[4]
+    if slots is not None:
+        _need(slots, "slots", torch.int32, (T,), dev)
+    q = torch.empty((T, Hq, Dc), dtype=qkv.dtype, device=dev)
+    _check(lib.qe_qkv_conv_rope_store(qkv.data_ptr(), conv_w.data_ptr(), _ptr(state), tok_seq.data_ptr(),
+                                      positions.data_ptr(), _ptr(inv_freq), _ptr(slots), q.data_ptr(), cache.data_ptr(),
+                                      T, Hq, Hkv, Dk, Dv, Dc, P, taps, rot, int(bool(single_rows)), _DT[qkv.dtype],
+                                      _stream()), "qkv_conv_rope_store")
+    return q
+
+
 def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor,
-                w_down: torch.Tensor, limit: float, slope: float, interleaved: bool = False,
-                algo: int = ALGO_AUTO) -> torch.Tensor:
+                w_down: torch.Tensor, limit: float = 0.0, slope: float = 1.0, interleaved: bool = False,
+                algo: int = ALGO_AUTO, act: str = "gated", identity: int = 0) -> torch.Tensor:
     """The chosen experts' outputs, weighted: float32 [S, T, H] whose sum over S, in order, is the mixture's
     output (S = top: a token's choices in their order; or S = 1: already added up in that order).
     x [T, K]; w_gate_up [E, 2 F, K] (gate rows, then up rows; or, ``interleaved``, in alternating blocks of
     32 as interleave_gate_up lays them); w_down [E, H, F].  An expert: g = min(gate x, limit),
-    u = clamp(up x, -limit, limit), down (g sigmoid(slope g) (u + 1)).
+    u = clamp(up x, -limit, limit), down (g sigmoid(slope g) (u + 1)).  With ``act`` "relu_sq" the first
+    matrix is one [E, F, K] and an expert is down (relu(up x)^2).  ``identity``: so many more
+    experts, the ids E .. E + identity - 1, are the identity: their output is the token's row itself, times the weight.
 
     The (token, choice) pairs are grouped by expert on the device.  bfloat16 with many pairs: their rows are
     gathered side by side and both products run on the tiled kernel of the dense products, a tile of 128
@@ -1042,15 +1122,22 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gat
     _need(weights, "weights", torch.float32, (T, top), dev)
     _need(w_gate_up, "w_gate_up", x.dtype, (None, None, K), dev)
     E, F2 = w_gate_up.shape[0], w_gate_up.shape[1]
-    Fd = F2 // 2
+    if act not in ("gated", "relu_sq"):
+        raise KernelError(f"moe_experts: activation {act!r}")
+    single = act == "relu_sq"
+    first_mode = 2 if single else 1
+    Fd = F2 if single else F2 // 2
     _need(w_down, "w_down", x.dtype, (E, None, Fd), dev)
     Hout = w_down.shape[1]
-    if interleaved and Fd % 32:
+    if interleaved and (Fd % 32 or single):
         raise KernelError("moe_experts: interleaved gate|up rows come in blocks of 32")
+    identity = int(identity)
+    if identity < 0 or (identity and Hout != K):
+        raise KernelError("moe_experts: identity experts keep the width")
     n = T * top
     mfma = (x.dtype == torch.bfloat16 and algo != ALGO_GENERIC and lib.qe_moe_gemm_mfma_supported(K)
             and lib.qe_moe_gemm_mfma_supported(Fd))
-    tiled = mfma and interleaved and n >= 1024 and K >= 64 and Fd >= 64
+    tiled = mfma and (interleaved or single) and n >= 1024 and K >= 64 and Fd >= 64
     if tiled:
         tile_rows = lib.qe_gemm_mfma_grouped_tile_rows()
     elif mfma:
@@ -1060,19 +1147,26 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gat
     max_tiles = (n + tile_rows - 1) // tile_rows + min(E, n)
     meta = torch.empty(2 * n + 3 * max_tiles + 1, dtype=torch.int32, device=dev)
     perm, inv, tiles, n_tiles = meta[:n], meta[n:2 * n], meta[2 * n:2 * n + 3 * max_tiles], meta[2 * n + 3 * max_tiles:]
-    _check(lib.qe_moe_sort(ids.data_ptr(), n, E, tile_rows, perm.data_ptr(), inv.data_ptr(), tiles.data_ptr(),
+    # (identity experts are buckets of the sort like the others, behind them, and get no tiles)
+    _check(lib.qe_moe_sort(ids.data_ptr(), n, E + identity, E, tile_rows, perm.data_ptr(), inv.data_ptr(), tiles.data_ptr(),
                            n_tiles.data_ptr(), max_tiles, _stream()), "moe_sort")
+
+    def identity(parts_, rows_):
+        if identity:
+            _check(lib.qe_moe_identity(x.data_ptr(), ids.data_ptr(), weights.data_ptr(), inv.data_ptr(), _ptr(parts_),
+                                       _ptr(rows_), T, top, Hout, E, _DT[x.dtype], _stream()), "moe_identity")
     a = torch.empty((n, Fd), dtype=x.dtype, device=dev)
     if tiled:
         xs = torch.empty((n, K), dtype=x.dtype, device=dev)
         _check(lib.qe_moe_gather(x.data_ptr(), perm.data_ptr(), top, xs.data_ptr(), n, K, _DT[x.dtype], _stream()), "moe_gather")
         _check(lib.qe_gemm_mfma_grouped(xs.data_ptr(), w_gate_up.data_ptr(), a.data_ptr(), tiles.data_ptr(),
-                                        n_tiles.data_ptr(), max_tiles, 2 * Fd, K, 1, float(limit), float(slope), BF16,
-                                        _stream()), "grouped gemm (gate, up)")
+                                        n_tiles.data_ptr(), max_tiles, Fd if single else 2 * Fd, K, first_mode, float(limit),
+                                        float(slope), BF16, _stream()), "grouped gemm (gate, up)")
         y = torch.empty((n, Hout), dtype=torch.float32, device=dev)
         _check(lib.qe_gemm_mfma_grouped(a.data_ptr(), w_down.data_ptr(), y.data_ptr(), tiles.data_ptr(),
                                         n_tiles.data_ptr(), max_tiles, Hout, Fd, 0, 0.0, 1.0, F32, _stream()),
                "grouped gemm (down)")
+        identity(None, y)
         out = torch.empty((1, T, Hout), dtype=torch.float32, device=dev)
         _check(lib.qe_moe_combine(y.data_ptr(), inv.data_ptr(), weights.data_ptr(), out.data_ptr(), T, top, Hout,
                                   _stream()), "moe_combine")
@@ -1081,15 +1175,17 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gat
     if mfma:
         _check(lib.qe_moe_gemm_mfma(x.data_ptr(), perm.data_ptr(), top, w_gate_up.data_ptr(), a.data_ptr(), None,
                                     tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, tile_rows, T, Fd, K, float(limit),
-                                    float(slope), 1, int(interleaved), _stream()), "moe_gemm (gate, up; mfma)")
+                                    float(slope), first_mode, int(interleaved), _stream()), "moe_gemm (gate, up; mfma)")
         _check(lib.qe_moe_gemm_mfma(a.data_ptr(), perm.data_ptr(), top, w_down.data_ptr(), parts.data_ptr(),
                                     weights.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, tile_rows, T,
                                     Hout, Fd, 0.0, 0.0, 0, 0, _stream()), "moe_gemm (down; mfma)")
+        identity(parts, None)
         return parts
     _check(lib.qe_moe_gemm(x.data_ptr(), perm.data_ptr(), top, w_gate_up.data_ptr(), a.data_ptr(), None,
-                           tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, T, Fd, K, float(limit), float(slope), 1,
+                           tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, T, Fd, K, float(limit), float(slope), first_mode,
                            int(interleaved), _DT[x.dtype], _DT[w_gate_up.dtype], _stream()), "moe_gemm (gate, up)")
     _check(lib.qe_moe_gemm(a.data_ptr(), perm.data_ptr(), top, w_down.data_ptr(), parts.data_ptr(), weights.data_ptr(),
                            tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, T, Hout, Fd, 0.0, 0.0, 0, 0,
                            _DT[x.dtype], _DT[w_down.dtype], _stream()), "moe_gemm (down)")
+    identity(parts, None)
     return parts

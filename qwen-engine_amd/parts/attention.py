@@ -278,4 +278,120 @@ class PagedAttention:
         return ops.gemm(o, self.w_o)
 
 
+def common_head_dim(k_dim: int, v_dim: int) -> int:
+    """The one head size under which keys and values of different sizes share the paged cache and the attention
+    kernels (zeros beyond a head's own numbers): 64 or 128, which the matrix-unit kernels take, else the next
+    multiple of 16."""
+    m = max(int(k_dim), int(v_dim))
+    if m <= 64:
+        return 64
+    if m <= 128:
+        return 128
+    return (m + 15) // 16 * 16
+
+
+class ConvAttention(PagedAttention):
+    """Grouped-query attention with a short causal convolution over time on every channel of the projected q, k
+    and v (``ConvAttentionSpec``): one product for q | k | v with the biases, then one kernel that convolves (a
+    request's last ``conv_taps - 1`` projected rows are its state), rotates the first numbers of every q and k head
+    and writes q and the cache, then the attention kernels of PagedAttention with the window's kept first keys and
+    the sink, then the output projection.  Keys and values of different sizes share the cache under one head size
+    (``common_head_dim``), and the output projection's columns beyond a value head's own numbers are zeros."""
+    takes_stream = False
+
+    def __init__(self, spec, hidden_size: int):
+        self.spec = spec
+        self.hidden = int(hidden_size)
+        self.hq, self.hkv = int(spec.num_heads), int(spec.num_kv_heads)
+        self.dk, self.dv = int(spec.head_dim), int(spec.v_head_dim)
+        self.d = common_head_dim(self.dk, self.dv)
+        if self.hq % self.hkv:
+            raise ValueError(f"{self.hq} query heads are no multiple of {self.hkv} key/value heads")
+        self.scale = float(spec.scale)
+        self.window = int(spec.window) if spec.window else 0
+        self.keep_first = int(spec.keep_first) if self.window else 0
+        self.sink = bool(spec.sink)
+        self.taps = int(spec.conv_taps)
+        self.position = build_part(spec.position, hidden_size) if spec.position is not None else None
+        self.w_qkv = self.b_qkv = self.w_o = self.conv_w = None
+
+    graph_safe = True        # every launch's grid follows the rows alone; the state is device memory
+
+    @staticmethod
+    def _channels(spec) -> int:
+        return spec.num_heads * spec.head_dim + spec.num_kv_heads * (spec.head_dim + spec.v_head_dim)
+
+    @staticmethod
+    def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
+        nq, nk, nv, no = spec.names
+        rows = {nq: spec.num_heads * spec.head_dim, nk: spec.num_kv_heads * spec.head_dim,
+                nv: spec.num_kv_heads * spec.v_head_dim}
+        t = {}
+        for name, n in rows.items():
+            t[name] = TensorInfo((n, hidden))
+            if spec.qkv_bias:
+                t[name + spec.bias_suffix] = TensorInfo((n,), "zeros", "vector")
+            if spec.conv_taps > 1:
+                t[name + spec.conv_suffix] = TensorInfo((n, int(spec.conv_taps)), "normal", "vector")
+        t[no] = TensorInfo((hidden, spec.num_heads * spec.v_head_dim))
+        return t
+
+    @staticmethod
+    def cache_need(spec) -> Optional[KVNeed]:
+        return KVNeed(num_kv_heads=spec.num_kv_heads, head_dim=common_head_dim(spec.head_dim, spec.v_head_dim),
+                      window=spec.window, keep_first=int(spec.keep_first) if spec.window else 0)
+
+    @staticmethod
+    def state_need(spec, hidden: int):
+        from ..cache.plan import StateNeed
+        taps = int(spec.conv_taps)
+        return StateNeed(shape=(taps - 1, ConvAttention._channels(spec)), dtype="float32") if taps > 1 else None
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        s = self.spec
+        nq, nk, nv, no = s.names
+        mats = [tensors[nq], tensors[nk], tensors[nv]]
+        if len({m.dtype for m in mats}) > 1:
+            mats = [m.float() for m in mats]
+        self.w_qkv = rt.place_matrix(torch.cat(mats, dim=0))
+        if s.qkv_bias:
+            self.b_qkv = rt.place_vector(torch.cat([tensors[n + s.bias_suffix].float() for n in (nq, nk, nv)]))
+        if self.taps > 1:
+            self.conv_w = rt.place_vector(torch.cat([tensors[n + s.conv_suffix].float() for n in (nq, nk, nv)], dim=0))
+        else:
+            self.conv_w = torch.ones((self._channels(s), 1), dtype=torch.float32, device=rt.device)
+        # the output projection against heads of the common size: zero columns beyond a value head's own numbers
+        w_o = tensors[no]
+        padded = torch.zeros((self.hidden, self.hq, self.d), dtype=w_o.dtype)
+        padded[:, :, :self.dv] = w_o.view(self.hidden, self.hq, self.dv)
+        self.w_o = rt.place_matrix(padded.view(self.hidden, self.hq * self.d))
+        if self.position is not None:
+            self.position.load({}, rt)
+
+    def forward(self, x: torch.Tensor, ctx, binding: CacheBinding) -> torch.Tensor:
+        """x [T, H] in the activation type.  Returns the mixer's output [T, H], or float32 partial products
+        [S, T, H] of it."""
+        if binding.kv is None:
+            raise RuntimeError("attention was given no cache")
+        if self.taps > 1 and binding.state is None:
+            raise RuntimeError("the convolution was given no state")
+        T, g, cache = x.shape[0], binding.group, binding.kv
+        qkv = ops.gemm(x, self.w_qkv, self.b_qkv)
+        # (a step in which every request brings one token: convolution and the state's shift in one launch)
+        single = all(s.q_len == 1 for s in ctx.seqs) and len(ctx.seqs) == T
+        q = ops.qkv_conv_rope_store(qkv, self.conv_w, binding.state, ctx.tok_seq, ctx.positions,
+                                    self.position.inv_freq() if self.position is not None else None,
+                                    ctx.slots[g] if binding.write else None, cache, self.hq, self.hkv, self.dk, self.dv,
+                                    single_rows=single)
+        ex = self._extras(ctx)
+        o = ops.attention(q, cache, ctx.positions, ctx.tok_seq, ctx.block_tables[g], self.scale, self.window,
+                          dec_tokens=ex["dec_tokens"], max_dec_position=ex["max_dec_position"],
+                          other_tokens=ex["other_tokens"],
+                          other_tiles=self._other_tiles(ctx) if ex["other_tokens"] is not None else None,
+                          max_other_keys=ex.get("max_other_keys", 0), other_keys_row=ex.get("other_keys_row"),
+                          shared_keys=ctx.shared_keys, keep_first=self.keep_first, sink=self.sink)
+        return self._project_out(o.view(T, self.hq * self.d))
+
+
 register_part("paged_attention", PagedAttention)
+register_part("conv_attention", ConvAttention)

@@ -187,5 +187,68 @@ class PostNormBlock:
         return None
 
 
+class ParallelBlock:
+    """n = norm(x); x <- x + (mixer(n) + ffn(n)): one norm, whose output both branches read, and one residual
+    sum in 32-bit.  The norm also adds what the block before left to be added (fused, as in PreNormBlock); the
+    mixer's output is added to the stream here, the feed-forward's is handed on for the next norm to add."""
+
+    def __init__(self, spec, hidden_size: int):
+        self.spec = spec
+        self.hidden = int(hidden_size)
+        self.norm = build_part(spec.norm, hidden_size)
+        self.mixer = build_part(spec.mixer, hidden_size)
+        self.ffn = build_part(spec.ffn, hidden_size) if spec.ffn is not None else None
+
+    def parts(self):
+        return tuple(p for p in (self.norm, self.mixer, self.ffn) if p is not None)
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(p, "graph_safe", True) for p in self.parts())
+
+    @property
+    def graph_safe_with_state(self) -> bool:
+        return getattr(self.mixer, "graph_safe", False) is True
+
+    @staticmethod
+    def _named(spec):
+        n_norm, n_mix, n_ffn = spec.names
+        out = [(n_norm, spec.norm), (n_mix, spec.mixer)]
+        if spec.ffn is not None:
+            out.append((n_ffn, spec.ffn))
+        return out
+
+    @staticmethod
+    def cache_needs(spec, hidden: int):
+        cls = part_class(spec.mixer.kind)
+        kv = cls.cache_need(spec.mixer) if hasattr(cls, "cache_need") else None
+        state = cls.state_need(spec.mixer, hidden) if hasattr(cls, "state_need") else None
+        return [(kv, state)]
+
+    @staticmethod
+    def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
+        out: Dict[str, TensorInfo] = {}
+        for name, sub in ParallelBlock._named(spec):
+            for rel, info in part_class(sub.kind).expected_tensors(sub, hidden).items():
+                out[join_name(name, rel)] = info
+        return out
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        for (name, sub), part in zip(self._named(self.spec), self.parts()):
+            names = type(part).expected_tensors(sub, self.hidden)
+            part.load(named_tensors(tensors, name, names), rt)
+
+    def forward(self, h, pending: Optional[torch.Tensor], ctx, bindings):
+        stream = h if isinstance(h, Stream) else Stream(h)
+        n = self.norm.forward(stream.h, ctx.rt, delta=pending)
+        a = self.mixer.forward(n, ctx, bindings[0])
+        if self.ffn is None:
+            return a
+        y = self.ffn.forward(n, ctx)
+        ops.residual_add(stream.h, a)
+        return y
+
+
 register_part("prenorm_block", PreNormBlock)
+register_part("parallel_block", ParallelBlock)
 register_part("postnorm_block", PostNormBlock)

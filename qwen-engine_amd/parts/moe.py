@@ -91,5 +91,53 @@ class GroupedMoE:
         return ops.moe_experts(x, ids, weights, self.w_gate_up, self.w_down, s.limit, s.slope, interleaved=self.interleaved)
 
 
+class BiasedMoE:
+    """A mixture of squared-relu experts with identity experts (``BiasedMoESpec``): router logits in 32-bit, softmax
+    over experts and identity experts together, the choice by score + correction, weights from the scores alone,
+    renormalised and scaled (``ops.moe_route_biased``); then the chosen experts' two products over the (token,
+    choice) pairs grouped by expert on the device, a pair that chose an identity expert contributing its token's
+    row itself (``ops.moe_experts``).  The output is float32 [top, T, H] or [1, T, H], as GroupedMoE's."""
+    graph_safe = True
+
+    def __init__(self, spec, hidden_size: int):
+        self.spec = spec
+        self.hidden = int(hidden_size)
+        self.e, self.ident, self.top, self.inter = (int(spec.num_experts), int(spec.num_identity), int(spec.top),
+                                                    int(spec.intermediate_size))
+        self.w_router = self.correction = self.w_up = self.w_down = None
+
+    @staticmethod
+    def expected_tensors(spec, hidden: int) -> Dict[str, TensorInfo]:
+        f, outs = spec.intermediate_size, spec.num_experts + spec.num_identity
+        t = {"router": TensorInfo((outs, hidden)), "correction": TensorInfo((outs,), "zeros", "vector")}
+        for e in range(spec.num_experts):
+            t[f"e{e}.up"] = TensorInfo((f, hidden))
+            t[f"e{e}.down"] = TensorInfo((hidden, f))
+        return t
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        self.w_router = rt.place_matrix(tensors["router"])
+        self.correction = rt.place_vector(tensors["correction"])
+        first = tensors["e0.up"]
+        dt = torch.float32 if rt.dtype == torch.float32 or first.dtype == torch.float32 else torch.bfloat16
+        self.w_up = torch.empty((self.e, self.inter, self.hidden), dtype=dt, device=rt.device)
+        self.w_down = torch.empty((self.e, self.hidden, self.inter), dtype=dt, device=rt.device)
+        for e in range(self.e):           # an expert at a time: the host never holds more
+            self.w_up[e].copy_(tensors[f"e{e}.up"])
+            self.w_down[e].copy_(tensors[f"e{e}.down"])
+
+    def active_weight_bytes(self, tokens: int) -> int:
+        """Bytes of expert weights that a step of ``tokens`` tokens reads at most."""
+        per = (self.w_up[0].numel() + self.w_down[0].numel()) * self.w_down.element_size()
+        return min(self.e, tokens * self.top) * per + self.w_router.numel() * self.w_router.element_size()
+
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        s = self.spec
+        logits = ops.gemm(x, self.w_router, out_dtype=torch.float32)
+        ids, weights = ops.moe_route_biased(logits, self.correction, s.top, s.route_scale)
+        return ops.moe_experts(x, ids, weights, self.w_up, self.w_down, act="relu_sq", identity=self.ident)
+
+
 register_part("polynorm_mlp", PolyNormMLP)
+register_part("biased_moe", BiasedMoE)
 register_part("grouped_moe", GroupedMoE)

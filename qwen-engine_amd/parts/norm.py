@@ -61,5 +61,35 @@ class ScalarRMSNorm:
         return ops.postnorm(x, delta, alpha, self.gain, self.eps, rt.dtype)
 
 
+class BareRMSNorm(RMSNorm):
+    """RMSNorm whose weight tensor carries the part's own name (named "" inside the part)."""
+
+    @staticmethod
+    def expected_tensors(spec, size: int) -> Dict[str, TensorInfo]:
+        return {"": TensorInfo((size,), "ones", "vector")}
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        self.weight = rt.place_vector(tensors[""])
+
+
+class StreamScale:
+    """Multiplies the 32-bit stream right after the embedding by one number."""
+
+    def __init__(self, spec, hidden_size: int = 0):
+        self.scale = float(spec.scale)
+
+    @staticmethod
+    def expected_tensors(spec, hidden_size: int) -> Dict[str, TensorInfo]:
+        return {}
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        pass
+
+    def forward(self, h: torch.Tensor, ctx) -> None:
+        ops.scale_(h, self.scale)
+
+
 register_part("rmsnorm", RMSNorm)
+register_part("rmsnorm_bare", BareRMSNorm)
+register_part("stream_scale", StreamScale)
 register_part("rmsnorm_scalar", ScalarRMSNorm)
