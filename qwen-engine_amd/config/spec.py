@@ -163,7 +163,7 @@ class RopeHalfAnglesSpec:
 @dataclass(frozen=True)
 class ConvAttentionSpec:
     """Grouped-query attention whose projected queries, keys and values (with biases if ``qkv_bias``) each pass
-    a causal convolution of ``conv_taps`` taps over time on every channel before q and k are rotated.  Keys have
+    a causal convolution of ``conv_taps`` taps over time on every channel before q and k are rotated (0: none).  Keys have
     ``head_dim`` numbers, values ``v_head_dim``.  ``window`` None: all earlier keys; else the last ``window`` keys
     (the query's own included) and, wherever the window stands, the request's first ``keep_first`` keys.
     ``sink``: the softmax's denominator has a 1 added (one more entry of score 0 that carries no value).
@@ -174,7 +174,7 @@ class ConvAttentionSpec:
     head_dim: int
     v_head_dim: int
     scale: float
-    conv_taps: int = 1
+    conv_taps: int = 0
     qkv_bias: bool = False
     window: Optional[int] = None
     keep_first: int = 0

@@ -331,7 +331,7 @@ class ConvAttention(PagedAttention):
             t[name] = TensorInfo((n, hidden))
             if spec.qkv_bias:
                 t[name + spec.bias_suffix] = TensorInfo((n,), "zeros", "vector")
-            if spec.conv_taps > 1:
+            if spec.conv_taps >= 1:
                 t[name + spec.conv_suffix] = TensorInfo((n, int(spec.conv_taps)), "normal", "vector")
         t[no] = TensorInfo((hidden, spec.num_heads * spec.v_head_dim))
         return t
@@ -356,9 +356,9 @@ class ConvAttention(PagedAttention):
         self.w_qkv = rt.place_matrix(torch.cat(mats, dim=0))
         if s.qkv_bias:
             self.b_qkv = rt.place_vector(torch.cat([tensors[n + s.bias_suffix].float() for n in (nq, nk, nv)]))
-        if self.taps > 1:
+        if self.taps >= 1:
             self.conv_w = rt.place_vector(torch.cat([tensors[n + s.conv_suffix].float() for n in (nq, nk, nv)], dim=0))
-        else:
+        else:                                              # no convolution: one tap of weight 1
             self.conv_w = torch.ones((self._channels(s), 1), dtype=torch.float32, device=rt.device)
         # the output projection against heads of the common size: zero columns beyond a value head's own numbers
         w_o = tensors[no]

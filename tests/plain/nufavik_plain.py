@@ -94,10 +94,10 @@ def attention(h: torch.Tensor, pos: torch.Tensor, w: Dict[str, torch.Tensor], pr
     size, keep = int(m["mask"]["size"]), int(m["mask"]["keep_first"])
     scale = float(m["scale"])
     out = torch.zeros(T, H, Dv, dtype=h.dtype)
-    for hh in range(H):
-        g = hh // (H // G)
-        for i in range(T):
-            js = [j for j in range(T) if sees(int(pos[i]), int(pos[j]), size, keep)]
+    for i in range(T):
+        js = [j for j in range(T) if sees(int(pos[i]), int(pos[j]), size, keep)]
+        for hh in range(H):
+            g = hh // (H // G)
             s = torch.stack([(q[i, hh] * k[j, g]).sum() * scale for j in js])
             p = softmax_with_sink(s)
             for pj, j in zip(p, js):
