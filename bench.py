@@ -35,7 +35,7 @@ Other sizes and workloads (not what the default line reports):
                             recorded graph of repetitions over weights that do not fit the caches, and its rate
                             against the nominal and the measured peaks (the counterpart of the reference's
                             per-operator benchmarks, src/layers/ops/linear.py:204-249)
-  --design zarorax          another design beside the closest Qwen3 model of equal sizes (width, layers, heads, and a
+  --design zarorax|nufavik  another design beside the closest Qwen3 model of equal sizes (width, layers, heads, and a
                             feed-forward as wide as the experts a token uses): prefill (one prompt of --prefill-tokens
                             in one step) and decode (batch 1 and --batch at --context) of both, at the sizes of
                             --design-sizes (small, medium); one JSON line of its own.  The default line is unchanged.
@@ -94,7 +94,7 @@ def parse():
                     help="run steps of single new tokens beside a prompt portion as they come, not from a recorded graph")
     ap.add_argument("--requests", type=int, default=None, help="requests of the serving workloads")
     ap.add_argument("--kernels", action="store_true", help="time each kernel of a layer alone over a range of rows")
-    ap.add_argument("--design", default=None, choices=["zarorax"],
+    ap.add_argument("--design", default=None, choices=["zarorax", "nufavik"],
                     help="measure this design beside the closest Qwen3 model of equal sizes instead of the default workload")
     ap.add_argument("--design-sizes", default="small,medium", help="which of the design's sizes (small, medium), with commas")
     ap.add_argument("--warmup-passes", type=int, default=2,
@@ -364,8 +364,29 @@ def zarorax_config(z, layers, vocab):
             "canon": {"taps": 4}, "layers": ls}
 
 
+# Layer sizes for --design nufavik: (width, query heads, key/value heads, key size, value size, taps, window, kept first
+# keys, rotated numbers, experts, identity experts, chosen, expert ff)
+NUFAVIK_SIZES = {
+    "small": dict(width=1024, heads=16, kv_heads=4, dim=64, vdim=64, conv=4, window=1024, keep_first=16, rot_dims=32,
+                  experts=32, identity=4, top=4, expert_ff=768),
+    "medium": dict(width=2048, heads=16, kv_heads=4, dim=128, vdim=128, conv=4, window=1024, keep_first=16, rot_dims=64,
+                   experts=32, identity=4, top=4, expert_ff=1024),
+}
+
+
+def nufavik_config(z, layers, vocab):
+    layer = {"type": "attention",
+             "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"], "conv": z["conv"],
+                       "scale": z["dim"] ** -0.5, "mask": {"size": z["window"], "keep_first": z["keep_first"]},
+                       "rot": {"base": 1000000.0, "dims": z["rot_dims"]}},
+             "mlp": {"kind": "moe", "expert": {"ff": z["expert_ff"]},
+                     "router": {"experts": z["experts"], "identity": z["identity"], "top": z["top"], "scale": 1.5}}}
+    return {"architecture": "Nufavik", "vocab": vocab, "width": z["width"], "embedding": {"scale": 0.5}, "norm": {"eps": 1e-5},
+            "layers": [layer] * layers}
+
+
 def design_compare(args) -> int:
-    """Prefill and decode of the Zarorax design beside the Qwen3 model of equal sizes, through the same step
+    """Prefill and decode of another design beside the Qwen3 model of equal sizes, through the same step
     function.  A "step" is one decode step; the line's value is the design's decode rate at --batch, first size."""
     import torch
     from qwen_engine_amd.config import config_from_dict
@@ -429,21 +450,29 @@ def design_compare(args) -> int:
         return res
 
     out = {}
+    design = args.design
+    title = design.capitalize()
     for name in [n for n in args.design_sizes.split(",") if n]:
-        z = ZARORAX_SIZES[name]
-        zcfg = config_from_dict(zarorax_config(z, layers, V))
+        if design == "nufavik":
+            z = NUFAVIK_SIZES[name]
+            zcfg = config_from_dict(nufavik_config(z, layers, V))
+            kv_heads, head_dim = z["kv_heads"], max(z["dim"], z["vdim"])
+        else:
+            z = ZARORAX_SIZES[name]
+            zcfg = config_from_dict(zarorax_config(z, layers, V))
+            kv_heads, head_dim = z["heads"] // 4, 128
         qcfg = config_from_dict(dict(QWEN3_0_6B, vocab_size=V, hidden_size=z["width"], intermediate_size=z["top"] * z["expert_ff"],
-                                     num_hidden_layers=layers, num_attention_heads=z["heads"], num_key_value_heads=z["heads"] // 4,
-                                     head_dim=128, tie_word_embeddings=False))
-        out[name] = {"sizes": dict(z, layers=layers, vocab=V), "zarorax": measure(zcfg), "qwen3": measure(qcfg)}
+                                     num_hidden_layers=layers, num_attention_heads=z["heads"], num_key_value_heads=kv_heads,
+                                     head_dim=head_dim, tie_word_embeddings=False))
+        out[name] = {"sizes": dict(z, layers=layers, vocab=V), design: measure(zcfg), "qwen3": measure(qcfg)}
         print(f"[bench] {name}: {out[name]}", file=sys.stderr, flush=True)
     first = next(iter(out.values()))
-    line = {"metric": f"decode tok/s @ batch {args.batch} (Zarorax, context {args.context}) beside Qwen3 of equal sizes",
-            "value": first["zarorax"][f"decode_b{args.batch}_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
-            "warmup": args.warmup, "ms_per_step": first["zarorax"][f"decode_b{args.batch}_ms_per_step"],
+    line = {"metric": f"decode tok/s @ batch {args.batch} ({title}, context {args.context}) beside Qwen3 of equal sizes",
+            "value": first[design][f"decode_b{args.batch}_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": first[design][f"decode_b{args.batch}_ms_per_step"],
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
             "data": "synthetic: random weights, uniform-random token ids",
-            "config": {"model": "Zarorax and Qwen3 layer sizes (random weights)", "global_batch": args.batch,
+            "config": {"model": f"{title} and Qwen3 layer sizes (random weights)", "global_batch": args.batch,
                        "seq_len": args.context, "prefill_tokens": args.prefill_tokens, "page_size": P, "parallelism": "single GPU"},
             "designs": out}
     print(json.dumps(line), flush=True)

@@ -245,6 +245,9 @@ class ParallelBlock:
         if self.ffn is None:
             return a
         y = self.ffn.forward(n, ctx)
+        if a.dim() == 3 and y.dim() == 3 and a.dtype == y.dtype:
+            # both branches left 32-bit parts (few rows): one list of parts, added in order by the next norm
+            return torch.cat([a, y], dim=0)
         ops.residual_add(stream.h, a)
         return y
 

@@ -1159,7 +1159,7 @@ def test_float32_attention_on_the_matrix_units(ops, hq, hkv, d, page, window):
     from qwen_engine_amd.kernels.ops import load_library, _DT
     lib = load_library()
     rc = lib.qe_attention(q_all.data_ptr(), part.data_ptr(), args[1].data_ptr(), args[2].data_ptr(), args[3].data_ptr(),
-                          args[4].data_ptr(), args[4].shape[1], rows.data_ptr(), 4, hq, hkv, d, page, scale, window, 0,
+                          args[4].data_ptr(), args[4].shape[1], rows.data_ptr(), 4, hq, hkv, d, page, scale, window, 0, 0, 0,
                           torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     torch.cuda.synchronize()
