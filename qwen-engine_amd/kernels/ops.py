@@ -76,7 +76,7 @@ def load_library():
         "qe_gemm_partial_preferred": [i32, i32, i32, i32, i32],
         "qe_gemm_branch_splits": [i32, i32, i32, i32, i32],
         "qe_attention": [vp, vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, i32, vp],
-        "qe_qkv_conv_rope_store": [vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, vp],
+        "qe_qkv_conv_rope_store": [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, vp],
         "qe_scale_f32": [vp, i64, f32, vp],
         "qe_moe_route_biased": [vp, vp, vp, vp, i32, i32, i32, f32, vp],
         "qe_moe_identity": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp],
@@ -1058,14 +1058,15 @@ def scale_(x: torch.Tensor, s: float) -> None:
 def qkv_conv_rope_store(qkv: torch.Tensor, conv_w: torch.Tensor, state: Optional[torch.Tensor], tok_seq: torch.Tensor,
                         positions: torch.Tensor, inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor],
                         cache: torch.Tensor, num_heads: int, num_kv_heads: int, k_dim: int, v_dim: int,
-                        single_rows: bool = False) -> torch.Tensor:
+                        single_rows: bool = False, conv_w_t: Optional[torch.Tensor] = None) -> torch.Tensor:
     """What stands between a q|k|v projection and the attention where q, k and v each pass a short causal
     convolution over time and q and k are then rotated on their first numbers.  qkv [T, Hq Dk + Hkv Dk + Hkv Dv];
     conv_w float32 [that many, taps]; state float32 [slots, taps - 1, that many] (row tok_seq[t]: the request's last
     projected rows; None for one tap), brought up to date; inv_freq float32 [rotated numbers / 2] or None.
     cache [pages, 2, Hkv, P, Dc] with Dc >= Dk, Dv: keys and values go to slots[t] (negative or no slots:
     nowhere), zeros beyond a head's own numbers.  Returns q [T, Hq, Dc], padded likewise.  The rows of a request
-    are consecutive; ``single_rows``: no two rows belong to the same request (one launch)."""
+    are consecutive; ``single_rows``: no two rows belong to the same request (one launch).  ``conv_w_t``: conv_w
+    transposed, float32 [taps, that many], for the kernel of many rows (eight channels a thread)."""
     lib = load_library()
     _need(qkv, "qkv", _ACT, (None, None))
     T, C = qkv.shape
@@ -1089,8 +1090,10 @@ def qkv_conv_rope_store(qkv: torch.Tensor, conv_w: torch.Tensor, state: Optional
     P, Dc = cache.shape[3], cache.shape[4]
     if slots is not None:
         _need(slots, "slots", torch.int32, (T,), dev)
+    if conv_w_t is not None:
+        _need(conv_w_t, "conv_w_t", torch.float32, (taps, C), dev)
     q = torch.empty((T, Hq, Dc), dtype=qkv.dtype, device=dev)
-    _check(lib.qe_qkv_conv_rope_store(qkv.data_ptr(), conv_w.data_ptr(), _ptr(state), tok_seq.data_ptr(),
+    _check(lib.qe_qkv_conv_rope_store(qkv.data_ptr(), conv_w.data_ptr(), _ptr(conv_w_t), _ptr(state), tok_seq.data_ptr(),
                                       positions.data_ptr(), _ptr(inv_freq), _ptr(slots), q.data_ptr(), cache.data_ptr(),
                                       T, Hq, Hkv, Dk, Dv, Dc, P, taps, rot, int(bool(single_rows)), _DT[qkv.dtype],
                                       _stream()), "qkv_conv_rope_store")

@@ -313,7 +313,7 @@ class ConvAttention(PagedAttention):
         self.sink = bool(spec.sink)
         self.taps = int(spec.conv_taps)
         self.position = build_part(spec.position, hidden_size) if spec.position is not None else None
-        self.w_qkv = self.b_qkv = self.w_o = self.conv_w = None
+        self.w_qkv = self.b_qkv = self.w_o = self.conv_w = self.conv_w_t = None
 
     graph_safe = True        # every launch's grid follows the rows alone; the state is device memory
 
@@ -360,6 +360,7 @@ class ConvAttention(PagedAttention):
             self.conv_w = rt.place_vector(torch.cat([tensors[n + s.conv_suffix].float() for n in (nq, nk, nv)], dim=0))
         else:                                              # no convolution: one tap of weight 1
             self.conv_w = torch.ones((self._channels(s), 1), dtype=torch.float32, device=rt.device)
+        self.conv_w_t = self.conv_w.t().contiguous()      # [taps, channels]: what the kernel for many rows reads
         # the output projection against heads of the common size: zero columns beyond a value head's own numbers
         w_o = tensors[no]
         padded = torch.zeros((self.hidden, self.hq, self.d), dtype=w_o.dtype)
@@ -382,7 +383,7 @@ class ConvAttention(PagedAttention):
         q = ops.qkv_conv_rope_store(qkv, self.conv_w, binding.state, ctx.tok_seq, ctx.positions,
                                     self.position.inv_freq() if self.position is not None else None,
                                     ctx.slots[g] if binding.write else None, cache, self.hq, self.hkv, self.dk, self.dv,
-                                    single_rows=single)
+                                    single_rows=single, conv_w_t=self.conv_w_t)
         ex = self._extras(ctx)
         o = ops.attention(q, cache, ctx.positions, ctx.tok_seq, ctx.block_tables[g], self.scale, self.window,
                           dec_tokens=ex["dec_tokens"], max_dec_position=ex["max_dec_position"],
