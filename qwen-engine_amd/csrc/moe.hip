@@ -169,9 +169,9 @@ extern "C" int qe_moe_route_biased(const float* logits, const float* correction,
 // One block per (token, choice) pair that chose an identity expert (id >= E_real): its part of the output is the
 // token's row itself.  parts != null: parts[j][t] = weight * x[t] (32-bit); else y[inv[pair]] = x[t] (32-bit), for a
 // caller that weighs and adds the sorted rows afterwards.
-template <typename TA>
+template <typename TA, typename TY>
 __global__ void moe_identity_kernel(const TA* __restrict__ x, const int* __restrict__ ids, const float* __restrict__ weights,
-                                    const int* __restrict__ inv, float* __restrict__ parts, float* __restrict__ y,
+                                    const int* __restrict__ inv, float* __restrict__ parts, TY* __restrict__ y,
                                     int T, int top, int H, int E_real) {
     const long pair = blockIdx.x;
     if (ids[pair] < E_real) return;
@@ -183,19 +183,21 @@ __global__ void moe_identity_kernel(const TA* __restrict__ x, const int* __restr
         float* dst = parts + ((long)j * T + t) * H;
         for (int c = threadIdx.x; c < H; c += blockDim.x) dst[c] = wgt * Elem<TA>::load(src + c);
     } else {
-        float* dst = y + (long)inv[pair] * H;
-        for (int c = threadIdx.x; c < H; c += blockDim.x) dst[c] = Elem<TA>::load(src + c);
+        TY* dst = y + (long)inv[pair] * H;
+        for (int c = threadIdx.x; c < H; c += blockDim.x) Elem<TY>::store(dst + c, Elem<TA>::load(src + c));
     }
 }
 
-extern "C" int qe_moe_identity(const void* x, const int* ids, const float* weights, const int* inv, float* parts, float* y,
-                               int T, int top, int H, int E_real, int dt_a, hipStream_t stream) {
+// y: sorted rows in x's type if y_as_x, else float
+extern "C" int qe_moe_identity(const void* x, const int* ids, const float* weights, const int* inv, float* parts, void* y,
+                               int T, int top, int H, int E_real, int dt_a, int y_as_x, hipStream_t stream) {
     QE_REQUIRE(T >= 0 && top > 0 && H > 0 && E_real >= 0, "moe_identity: bad sizes");
     QE_REQUIRE((parts != nullptr) != (y != nullptr), "moe_identity: parts or sorted rows, one of them");
     QE_REQUIRE(parts || inv, "moe_identity: sorted rows need the pairs' places");
     if (T == 0) return 0;
-    if (dt_a == QE_BF16) moe_identity_kernel<bf16_t><<<T * top, 256, 0, stream>>>((const bf16_t*)x, ids, weights, inv, parts, y, T, top, H, E_real);
-    else if (dt_a == QE_F32) moe_identity_kernel<float><<<T * top, 256, 0, stream>>>((const float*)x, ids, weights, inv, parts, y, T, top, H, E_real);
+    if (dt_a == QE_BF16 && y_as_x) moe_identity_kernel<bf16_t, bf16_t><<<T * top, 256, 0, stream>>>((const bf16_t*)x, ids, weights, inv, parts, (bf16_t*)y, T, top, H, E_real);
+    else if (dt_a == QE_BF16) moe_identity_kernel<bf16_t, float><<<T * top, 256, 0, stream>>>((const bf16_t*)x, ids, weights, inv, parts, (float*)y, T, top, H, E_real);
+    else if (dt_a == QE_F32) moe_identity_kernel<float, float><<<T * top, 256, 0, stream>>>((const float*)x, ids, weights, inv, parts, (float*)y, T, top, H, E_real);
     else QE_REQUIRE(false, "moe_identity: unknown type %d", dt_a);
     QE_LAUNCH_CHECK();
     return 0;
@@ -399,21 +401,25 @@ extern "C" int qe_moe_gather(const void* x, const int* perm, int top, void* xs, 
     return 0;
 }
 
-__global__ void moe_combine_kernel(const float* __restrict__ y, const int* __restrict__ inv, const float* __restrict__ weights,
+template <typename TY>
+__global__ void moe_combine_kernel(const TY* __restrict__ y, const int* __restrict__ inv, const float* __restrict__ weights,
                                    float* __restrict__ out, int top, int H) {
     const long t = blockIdx.x;
     for (int c = threadIdx.x; c < H; c += blockDim.x) {
         float a = 0.f;
-        for (int j = 0; j < top; ++j) a = fmaf(weights[t * top + j], y[(long)inv[t * top + j] * H + c], a);
+        for (int j = 0; j < top; ++j) a = fmaf(weights[t * top + j], Elem<TY>::load(y + (long)inv[t * top + j] * H + c), a);
         out[t * H + c] = a;
     }
 }
 
-extern "C" int qe_moe_combine(const float* y, const int* inv, const float* weights, float* out, int T, int top, int H,
-                              hipStream_t stream) {
+// y: the sorted rows, float or bfloat16 (dt_y); the sum is 32-bit either way
+extern "C" int qe_moe_combine(const void* y, const int* inv, const float* weights, float* out, int T, int top, int H,
+                              int dt_y, hipStream_t stream) {
     QE_REQUIRE(T >= 0 && top > 0 && H > 0, "moe_combine: bad sizes");
     if (T == 0) return 0;
-    moe_combine_kernel<<<T, 256, 0, stream>>>(y, inv, weights, out, top, H);
+    if (dt_y == QE_F32) moe_combine_kernel<float><<<T, 256, 0, stream>>>((const float*)y, inv, weights, out, top, H);
+    else if (dt_y == QE_BF16) moe_combine_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)y, inv, weights, out, top, H);
+    else QE_REQUIRE(false, "moe_combine: unknown type %d", dt_y);
     QE_LAUNCH_CHECK();
     return 0;
 }

@@ -79,7 +79,7 @@ def load_library():
         "qe_qkv_conv_rope_store": [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, vp],
         "qe_scale_f32": [vp, i64, f32, vp],
         "qe_moe_route_biased": [vp, vp, vp, vp, i32, i32, i32, f32, vp],
-        "qe_moe_identity": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, vp],
+        "qe_moe_identity": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp],
         "qe_argmax": [vp, vp, i32, i32, vp, i64, vp],
         "qe_argmax_static": [vp, vp, i32, i32, vp],
         "qe_sample": [vp, vp, vp, vp, i32, i32, vp],
@@ -98,7 +98,7 @@ def load_library():
         "qe_moe_sort": [vp, i32, i32, i32, i32, vp, vp, vp, vp, i32, vp],
         "qe_moe_gemm": [vp, vp, i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, f32, i32, i32, i32, i32, vp],
         "qe_moe_gather": [vp, vp, i32, vp, i32, i32, i32, vp],
-        "qe_moe_combine": [vp, vp, vp, vp, i32, i32, i32, vp],
+        "qe_moe_combine": [vp, vp, vp, vp, i32, i32, i32, i32, vp],
         "qe_gemm_mfma_grouped": [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, f32, i32, vp],
         "qe_gemm_mfma_grouped_tile_rows": [],
         "qe_moe_tile_rows": [],
@@ -1102,7 +1102,8 @@ def qkv_conv_rope_store(qkv: torch.Tensor, conv_w: torch.Tensor, state: Optional
 
 def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor,
                 w_down: torch.Tensor, limit: float = 0.0, slope: float = 1.0, interleaved: bool = False,
-                algo: int = ALGO_AUTO, act: str = "gated", identity: int = 0) -> torch.Tensor:
+                algo: int = ALGO_AUTO, act: str = "gated", identity: int = 0,
+                rows_dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """The chosen experts' outputs, weighted: float32 [S, T, H] whose sum over S, in order, is the mixture's
     output (S = top: a token's choices in their order; or S = 1: already added up in that order).
     x [T, K]; w_gate_up [E, 2 F, K] (gate rows, then up rows; or, ``interleaved``, in alternating blocks of
@@ -1110,6 +1111,9 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gat
     u = clamp(up x, -limit, limit), down (g sigmoid(slope g) (u + 1)).  With ``act`` "relu_sq" the first
     matrix is one [E, F, K] and an expert is down (relu(up x)^2).  ``identity``: so many more
     experts, the ids E .. E + identity - 1, are the identity: their output is the token's row itself, times the weight.
+    ``rows_dtype``: the element type in which the path of many pairs leaves an expert's output rows before they are
+    weighed and added in 32-bit (float32, or bfloat16 with bfloat16 operands: half the bytes of the largest tensor of
+    the mixture).
 
     The (token, choice) pairs are grouped by expert on the device.  bfloat16 with many pairs: their rows are
     gathered side by side and both products run on the tiled kernel of the dense products, a tile of 128
@@ -1157,7 +1161,9 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gat
     def identity(parts_, rows_):
         if identity:
             _check(lib.qe_moe_identity(x.data_ptr(), ids.data_ptr(), weights.data_ptr(), inv.data_ptr(), _ptr(parts_),
-                                       _ptr(rows_), T, top, Hout, E, _DT[x.dtype], _stream()), "moe_identity")
+                                       _ptr(rows_), T, top, Hout, E, _DT[x.dtype],
+                                       int(rows_ is not None and rows_.dtype == x.dtype and x.dtype != torch.float32),
+                                       _stream()), "moe_identity")
     a = torch.empty((n, Fd), dtype=x.dtype, device=dev)
     if tiled:
         xs = torch.empty((n, K), dtype=x.dtype, device=dev)
@@ -1165,14 +1171,16 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gat
         _check(lib.qe_gemm_mfma_grouped(xs.data_ptr(), w_gate_up.data_ptr(), a.data_ptr(), tiles.data_ptr(),
                                         n_tiles.data_ptr(), max_tiles, Fd if single else 2 * Fd, K, first_mode, float(limit),
                                         float(slope), BF16, _stream()), "grouped gemm (gate, up)")
-        y = torch.empty((n, Hout), dtype=torch.float32, device=dev)
+        if rows_dtype not in (torch.float32, torch.bfloat16):
+            raise KernelError(f"moe_experts: rows in {rows_dtype}")
+        y = torch.empty((n, Hout), dtype=rows_dtype, device=dev)
         _check(lib.qe_gemm_mfma_grouped(a.data_ptr(), w_down.data_ptr(), y.data_ptr(), tiles.data_ptr(),
-                                        n_tiles.data_ptr(), max_tiles, Hout, Fd, 0, 0.0, 1.0, F32, _stream()),
+                                        n_tiles.data_ptr(), max_tiles, Hout, Fd, 0, 0.0, 1.0, _DT[rows_dtype], _stream()),
                "grouped gemm (down)")
         identity(None, y)
         out = torch.empty((1, T, Hout), dtype=torch.float32, device=dev)
         _check(lib.qe_moe_combine(y.data_ptr(), inv.data_ptr(), weights.data_ptr(), out.data_ptr(), T, top, Hout,
-                                  _stream()), "moe_combine")
+                                  _DT[rows_dtype], _stream()), "moe_combine")
         return out
     parts = torch.empty((top, T, Hout), dtype=torch.float32, device=dev)
     if mfma:

@@ -135,7 +135,10 @@ class BiasedMoE:
         s = self.spec
         logits = ops.gemm(x, self.w_router, out_dtype=torch.float32)
         ids, weights = ops.moe_route_biased(logits, self.correction, s.top, s.route_scale)
-        return ops.moe_experts(x, ids, weights, self.w_up, self.w_down, act="relu_sq", identity=self.ident)
+        # (the experts' output rows of a long portion in the activation type: what a product leaves anywhere else;
+        # they are weighed and added in 32-bit)
+        return ops.moe_experts(x, ids, weights, self.w_up, self.w_down, act="relu_sq", identity=self.ident,
+                               rows_dtype=ctx.rt.dtype)
 
 
 register_part("polynorm_mlp", PolyNormMLP)

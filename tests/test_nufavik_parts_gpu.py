@@ -252,6 +252,8 @@ def test_squared_relu_experts_and_identity_experts_over_rows_grouped_on_the_devi
             e = int(ids[t, j])
             y = x[t].double() if e >= E else N.expert(x[t].double(), up[e].double(), down[e].double())
             want[t] += float(w[t, j]) * y
-    parts = ops().moe_experts(x.to(DEV), ids.to(DEV), w.to(DEV), up.to(DEV), down.to(DEV), act="relu_sq", identity=ident)
-    assert parts.dtype == torch.float32 and parts.shape[1:] == (T, H)
-    assert rel(parts.sum(0), want) < tol
+    for rows_dtype in {torch.float32, dtype}:             # (the element type of an expert's output rows where the pairs are many)
+        parts = ops().moe_experts(x.to(DEV), ids.to(DEV), w.to(DEV), up.to(DEV), down.to(DEV), act="relu_sq", identity=ident,
+                                  rows_dtype=rows_dtype)
+        assert parts.dtype == torch.float32 and parts.shape[1:] == (T, H)
+        assert rel(parts.sum(0), want) < tol
