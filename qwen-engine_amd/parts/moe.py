@@ -98,6 +98,7 @@ class BiasedMoE:
     choice) pairs grouped by expert on the device, a pair that chose an identity expert contributing its token's
     row itself (``ops.moe_experts``).  The output is float32 [top, T, H] or [1, T, H], as GroupedMoE's."""
     graph_safe = True
+    rows_in_activation_type = False
 
     def __init__(self, spec, hidden_size: int):
         self.spec = spec
@@ -135,10 +136,11 @@ class BiasedMoE:
         s = self.spec
         logits = ops.gemm(x, self.w_router, out_dtype=torch.float32)
         ids, weights = ops.moe_route_biased(logits, self.correction, s.top, s.route_scale)
-        # (the experts' output rows of a long portion in the activation type: what a product leaves anywhere else;
-        # they are weighed and added in 32-bit)
-        return ops.moe_experts(x, ids, weights, self.w_up, self.w_down, act="relu_sq", identity=self.ident,
-                               rows_dtype=ctx.rt.dtype)
+        # (rows_in_activation_type: the experts' output rows of a long portion in bfloat16 instead of 32-bit before
+        # they are weighed and added in 32-bit: 7 % less time for the down product and 18 % for the sum at 8192
+        # pairs of width 2048, for one more rounding of every expert's output; off)
+        rows = ctx.rt.dtype if self.rows_in_activation_type else torch.float32
+        return ops.moe_experts(x, ids, weights, self.w_up, self.w_down, act="relu_sq", identity=self.ident, rows_dtype=rows)
 
 
 register_part("polynorm_mlp", PolyNormMLP)
