@@ -107,53 +107,63 @@ extern "C" int qe_moe_route(const float* logits, int* ids, float* weights, int T
 }
 
 
-// One wave per token: softmax over all E experts, choice by score + correction, weights from the scores alone.
+// One token's routing by one wave: softmax over all E outputs, choice by score + correction, weights from the
+// scores alone.  sc: the wave's own 2 E + top floats of shared memory.  Every wave of the block calls it together
+// (the barriers are the block's); a wave without a token (z null) only keeps step.
+__device__ __forceinline__ void route_biased_token(const float* __restrict__ z, const float* __restrict__ correction,
+                                                   float* sc, int* __restrict__ ids, float* __restrict__ weights, int E,
+                                                   int top, float scale, int lane) {
+    float* ch = sc + E;
+    float* picked = ch + E;
+    if (z) {
+        float mx = -INFINITY;
+        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int e = lane; e < E; e += 64) {
+            const float ex = expf(z[e] - mx);
+            sc[e] = ex;
+            sum += ex;
+        }
+        sum = wave_sum(sum);
+        for (int e = lane; e < E; e += 64) {
+            float v = sc[e] / sum;
+            if (!(v == v)) v = 0.f;            // (a row of garbage still gets experts inside the table)
+            sc[e] = v;
+            float c = v + correction[e];
+            if (!(c == c)) c = 0.f;
+            ch[e] = c;
+        }
+    }
+    __syncthreads();
+    for (int r = 0; r < top; ++r) {
+        if (z) {
+            float bv = -INFINITY;
+            int bi = -1;
+            for (int e = lane; e < E; e += 64)
+                if (ch[e] > bv) { bv = ch[e]; bi = e; }
+            wave_argmax(bv, bi);
+            if (lane == 0) {
+                ids[r] = bi >= 0 ? bi : 0;
+                picked[r] = bi >= 0 ? sc[bi] : 0.f;
+                if (bi >= 0) ch[bi] = -INFINITY;
+            }
+        }
+        __syncthreads();
+    }
+    if (z && lane == 0) {
+        float tot = 0.f;
+        for (int r = 0; r < top; ++r) tot += picked[r];
+        for (int r = 0; r < top; ++r) weights[r] = picked[r] / (tot + 1e-20f) * scale;
+    }
+}
+
 __global__ __launch_bounds__(64) void moe_route_biased_kernel(const float* __restrict__ logits, const float* __restrict__ correction,
                                                               int* __restrict__ ids, float* __restrict__ weights, int E, int top,
                                                               float scale) {
     extern __shared__ float sc[];          // E scores, E choice scores, top chosen scores
-    float* ch = sc + E;
-    float* picked = ch + E;
     const long t = blockIdx.x;
-    const int lane = threadIdx.x;
-    const float* z = logits + t * E;
-    float mx = -INFINITY;
-    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
-    mx = wave_max(mx);
-    float sum = 0.f;
-    for (int e = lane; e < E; e += 64) {
-        const float ex = expf(z[e] - mx);
-        sc[e] = ex;
-        sum += ex;
-    }
-    sum = wave_sum(sum);
-    for (int e = lane; e < E; e += 64) {
-        float v = sc[e] / sum;
-        if (!(v == v)) v = 0.f;            // (a row of garbage still gets experts inside the table)
-        sc[e] = v;
-        float c = v + correction[e];
-        if (!(c == c)) c = 0.f;
-        ch[e] = c;
-    }
-    __syncthreads();
-    for (int r = 0; r < top; ++r) {
-        float bv = -INFINITY;
-        int bi = -1;
-        for (int e = lane; e < E; e += 64)
-            if (ch[e] > bv) { bv = ch[e]; bi = e; }
-        wave_argmax(bv, bi);
-        if (lane == 0) {
-            ids[t * top + r] = bi >= 0 ? bi : 0;
-            picked[r] = bi >= 0 ? sc[bi] : 0.f;
-            if (bi >= 0) ch[bi] = -INFINITY;
-        }
-        __syncthreads();
-    }
-    if (lane == 0) {
-        float tot = 0.f;
-        for (int r = 0; r < top; ++r) tot += picked[r];
-        for (int r = 0; r < top; ++r) weights[t * top + r] = picked[r] / (tot + 1e-20f) * scale;
-    }
+    route_biased_token(logits + t * E, correction, sc, ids + t * top, weights + t * top, E, top, scale, threadIdx.x);
 }
 
 extern "C" int qe_moe_route_biased(const float* logits, const float* correction, int* ids, float* weights, int T, int E,
@@ -205,12 +215,9 @@ extern "C" int qe_moe_identity(const void* x, const int* ids, const float* weigh
 
 // One block.  n = T * top pairs.  Only the first tile_experts experts get tiles (the others' pairs still get
 // their places in perm, behind them).
-__global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ ids, int n, int E, int tile_experts, int tile_rows,
-                                                        int* __restrict__ perm, int* __restrict__ inv,
-                                                        int* __restrict__ tiles, int* __restrict__ n_tiles) {
-    extern __shared__ int sm[];
-    int* counts = sm;
-    int* cursor = sm + E;
+__device__ __forceinline__ void sort_pairs(const int* ids, int n, int E, int tile_experts, int tile_rows,
+                                           int* __restrict__ perm, int* __restrict__ inv, int* __restrict__ tiles,
+                                           int* __restrict__ n_tiles, int* counts, int* cursor) {
     const int tid = threadIdx.x;
     for (int e = tid; e < E; e += blockDim.x) counts[e] = 0;
     __syncthreads();
@@ -238,6 +245,77 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ 
         perm[at] = i;
         if (inv) inv[i] = at;
     }
+}
+
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ ids, int n, int E, int tile_experts, int tile_rows,
+                                                        int* __restrict__ perm, int* __restrict__ inv,
+                                                        int* __restrict__ tiles, int* __restrict__ n_tiles) {
+    extern __shared__ int sm[];
+    sort_pairs(ids, n, E, tile_experts, tile_rows, perm, inv, tiles, n_tiles, sm, sm + E);
+}
+
+// A step of few tokens (T * top <= 1024 pairs): routing, sort and the identity experts' rows in one launch of one
+// block, where three launches cost three times a dependent kernel's few microseconds.  Wave w routes the tokens
+// w, w + 16, ...; the pairs' ids stay in shared memory for the sort; then every pair that chose an identity expert
+// gets its token's row, weighted, as its part.
+template <typename TA>
+__global__ __launch_bounds__(1024) void moe_front_small_kernel(
+    const float* __restrict__ logits, const float* __restrict__ correction, const TA* __restrict__ x, int* __restrict__ ids,
+    float* __restrict__ weights, int* __restrict__ perm, int* __restrict__ inv, int* __restrict__ tiles,
+    int* __restrict__ n_tiles, float* __restrict__ parts, int T, int H, int E, int E_real, int top, float scale, int tile_rows) {
+    extern __shared__ int sm[];
+    const int n = T * top;
+    int* ids_s = sm;                                     // n
+    float* w_s = (float*)(sm + n);                       // n
+    int* counts = sm + 2 * n;                            // E, then E cursors
+    float* wave_sc = (float*)(sm + 2 * n + 2 * E);       // 16 waves of 2 E + top
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    for (int t0 = 0; t0 < T; t0 += waves) {
+        const int t = t0 + wave;
+        route_biased_token(t < T ? logits + (long)t * E : nullptr, correction, wave_sc + (long)wave * (2 * E + top),
+                           ids_s + (t < T ? t : 0) * top, w_s + (t < T ? t : 0) * top, E, top, scale, lane);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        ids[i] = ids_s[i];
+        weights[i] = w_s[i];
+    }
+    sort_pairs(ids_s, n, E, E_real, tile_rows, perm, inv, tiles, n_tiles, counts, counts + E);
+    if (E_real < E) {
+        for (int i = 0; i < n; ++i) {
+            if (ids_s[i] < E_real) continue;
+            const int t = i / top, j = i - t * top;
+            const float wgt = w_s[i];
+            float* dst = parts + ((long)j * T + t) * H;
+            const TA* src = x + (long)t * H;
+            for (int c = threadIdx.x; c < H; c += blockDim.x) dst[c] = wgt * Elem<TA>::load(src + c);
+        }
+    }
+}
+
+extern "C" int qe_moe_front_small_supported(int T, int E, int top) {
+    return T > 0 && (long)T * top <= 1024 && ((long)2 * T * top + 2 * E + 16L * (2 * E + top)) * 4 <= 60000;
+}
+
+// logits float [T, E] (experts and identity experts together), correction [E]; ids, weights [T, top]; perm, inv
+// [T top]; tiles, n_tiles as qe_moe_sort leaves them for the first E_real experts; parts float [top, T, H]: the
+// parts of the pairs that chose an identity expert (E_real .. E - 1) are written, the others left.
+extern "C" int qe_moe_front_small(const float* logits, const float* correction, const void* x, int* ids, float* weights,
+                                  int* perm, int* inv, int* tiles, int* n_tiles, float* parts, int max_tiles, int T, int H,
+                                  int E, int E_real, int top, float scale, int tile_rows, int dt_a, hipStream_t stream) {
+    QE_REQUIRE(qe_moe_front_small_supported(T, E, top), "moe_front_small: %d tokens, %d outputs, top %d", T, E, top);
+    QE_REQUIRE(E_real >= 1 && E_real <= E && top <= E && tile_rows > 0 && H > 0, "moe_front_small: bad sizes");
+    const int n = T * top;
+    QE_REQUIRE(max_tiles >= (n + tile_rows - 1) / tile_rows + (E_real < n ? E_real : n), "moe_front_small: %d tiles may not be enough", max_tiles);
+    const size_t lds = ((size_t)2 * n + 2 * E + 16 * (2 * E + top)) * 4;
+    if (dt_a == QE_BF16)
+        moe_front_small_kernel<bf16_t><<<1, 1024, lds, stream>>>(logits, correction, (const bf16_t*)x, ids, weights, perm, inv, tiles, n_tiles, parts, T, H, E, E_real, top, scale, tile_rows);
+    else if (dt_a == QE_F32)
+        moe_front_small_kernel<float><<<1, 1024, lds, stream>>>(logits, correction, (const float*)x, ids, weights, perm, inv, tiles, n_tiles, parts, T, H, E, E_real, top, scale, tile_rows);
+    else
+        QE_REQUIRE(false, "moe_front_small: unknown type %d", dt_a);
+    QE_LAUNCH_CHECK();
+    return 0;
 }
 
 // inv (may be null): the sorted row of every pair, perm's inverse

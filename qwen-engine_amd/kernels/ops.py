@@ -79,6 +79,8 @@ def load_library():
         "qe_qkv_conv_rope_store": [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, vp],
         "qe_scale_f32": [vp, i64, f32, vp],
         "qe_moe_route_biased": [vp, vp, vp, vp, i32, i32, i32, f32, vp],
+        "qe_moe_front_small_supported": [i32, i32, i32],
+        "qe_moe_front_small": [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, i32, vp],
         "qe_moe_identity": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp],
         "qe_argmax": [vp, vp, i32, i32, vp, i64, vp],
         "qe_argmax_static": [vp, vp, i32, i32, vp],
@@ -1100,10 +1102,10 @@ def qkv_conv_rope_store(qkv: torch.Tensor, conv_w: torch.Tensor, state: Optional
     return q
 
 
-def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor,
+def moe_experts(x: torch.Tensor, ids: Optional[torch.Tensor], weights: Optional[torch.Tensor], w_gate_up: torch.Tensor,
                 w_down: torch.Tensor, limit: float = 0.0, slope: float = 1.0, interleaved: bool = False,
                 algo: int = ALGO_AUTO, act: str = "gated", identity: int = 0,
-                rows_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+                rows_dtype: torch.dtype = torch.float32, biased_route=None) -> torch.Tensor:
     """The chosen experts' outputs, weighted: float32 [S, T, H] whose sum over S, in order, is the mixture's
     output (S = top: a token's choices in their order; or S = 1: already added up in that order).
     x [T, K]; w_gate_up [E, 2 F, K] (gate rows, then up rows; or, ``interleaved``, in alternating blocks of
@@ -1113,7 +1115,9 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gat
     experts, the ids E .. E + identity - 1, are the identity: their output is the token's row itself, times the weight.
     ``rows_dtype``: the element type in which the path of many pairs leaves an expert's output rows before they are
     weighed and added in 32-bit (float32, or bfloat16 with bfloat16 operands: half the bytes of the largest tensor of
-    the mixture).
+    the mixture).  ``biased_route``: instead of ids and weights (both None), (logits float32 [T, E + identity],
+    correction float32 [E + identity], top, scale) for the routing of moe_route_biased: a step of few tokens then
+    routes, sorts and writes the identity experts' rows in one launch.
 
     The (token, choice) pairs are grouped by expert on the device.  bfloat16 with many pairs: their rows are
     gathered side by side and both products run on the tiled kernel of the dense products, a tile of 128
@@ -1124,9 +1128,17 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gat
     _need(x, "x", _ACT, (None, None))
     T, K = x.shape
     dev = x.device
-    _need(ids, "ids", torch.int32, (T, None), dev)
-    top = ids.shape[1]
-    _need(weights, "weights", torch.float32, (T, top), dev)
+    if biased_route is not None:
+        if ids is not None or weights is not None:
+            raise KernelError("moe_experts: ids and weights, or a route to compute them, not both")
+        r_logits, r_corr, top, r_scale = biased_route
+        top = int(top)
+        _need(r_logits, "logits", torch.float32, (T, None), dev)
+        _need(r_corr, "correction", torch.float32, (r_logits.shape[1],), dev)
+    else:
+        _need(ids, "ids", torch.int32, (T, None), dev)
+        top = ids.shape[1]
+        _need(weights, "weights", torch.float32, (T, top), dev)
     _need(w_gate_up, "w_gate_up", x.dtype, (None, None, K), dev)
     E, F2 = w_gate_up.shape[0], w_gate_up.shape[1]
     if act not in ("gated", "relu_sq"):
@@ -1154,12 +1166,30 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gat
     max_tiles = (n + tile_rows - 1) // tile_rows + min(E, n)
     meta = torch.empty(2 * n + 3 * max_tiles + 1, dtype=torch.int32, device=dev)
     perm, inv, tiles, n_tiles = meta[:n], meta[n:2 * n], meta[2 * n:2 * n + 3 * max_tiles], meta[2 * n + 3 * max_tiles:]
+    fused_front = False
+    parts = None
+    if biased_route is not None:
+        if r_logits.shape[1] != E + identity:
+            raise KernelError(f"moe_experts: {r_logits.shape[1]} router outputs for {E} experts and {identity} identity experts")
+        if not tiled and lib.qe_moe_front_small_supported(T, E + identity, top):
+            # few tokens: routing, sort and the identity experts' rows in one launch
+            ids = torch.empty((T, top), dtype=torch.int32, device=dev)
+            weights = torch.empty((T, top), dtype=torch.float32, device=dev)
+            parts = torch.empty((top, T, Hout), dtype=torch.float32, device=dev)
+            _check(lib.qe_moe_front_small(r_logits.data_ptr(), r_corr.data_ptr(), x.data_ptr(), ids.data_ptr(),
+                                          weights.data_ptr(), perm.data_ptr(), inv.data_ptr(), tiles.data_ptr(),
+                                          n_tiles.data_ptr(), parts.data_ptr(), max_tiles, T, Hout, E + identity, E, top,
+                                          float(r_scale), tile_rows, _DT[x.dtype], _stream()), "moe_front_small")
+            fused_front = True
+        else:
+            ids, weights = moe_route_biased(r_logits, r_corr, top, r_scale)
     # (identity experts are buckets of the sort like the others, behind them, and get no tiles)
-    _check(lib.qe_moe_sort(ids.data_ptr(), n, E + identity, E, tile_rows, perm.data_ptr(), inv.data_ptr(), tiles.data_ptr(),
-                           n_tiles.data_ptr(), max_tiles, _stream()), "moe_sort")
+    if not fused_front:
+        _check(lib.qe_moe_sort(ids.data_ptr(), n, E + identity, E, tile_rows, perm.data_ptr(), inv.data_ptr(), tiles.data_ptr(),
+                               n_tiles.data_ptr(), max_tiles, _stream()), "moe_sort")
 
     def identity(parts_, rows_):
-        if identity:
+        if identity and not fused_front:
             _check(lib.qe_moe_identity(x.data_ptr(), ids.data_ptr(), weights.data_ptr(), inv.data_ptr(), _ptr(parts_),
                                        _ptr(rows_), T, top, Hout, E, _DT[x.dtype],
                                        int(rows_ is not None and rows_.dtype == x.dtype and x.dtype != torch.float32),
@@ -1182,7 +1212,8 @@ def moe_experts(x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gat
         _check(lib.qe_moe_combine(y.data_ptr(), inv.data_ptr(), weights.data_ptr(), out.data_ptr(), T, top, Hout,
                                   _DT[rows_dtype], _stream()), "moe_combine")
         return out
-    parts = torch.empty((top, T, Hout), dtype=torch.float32, device=dev)
+    if parts is None:
+        parts = torch.empty((top, T, Hout), dtype=torch.float32, device=dev)
     if mfma:
         _check(lib.qe_moe_gemm_mfma(x.data_ptr(), perm.data_ptr(), top, w_gate_up.data_ptr(), a.data_ptr(), None,
                                     tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, tile_rows, T, Fd, K, float(limit),

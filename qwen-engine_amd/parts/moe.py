@@ -94,7 +94,8 @@ class GroupedMoE:
 class BiasedMoE:
     """A mixture of squared-relu experts with identity experts (``BiasedMoESpec``): router logits in 32-bit, softmax
     over experts and identity experts together, the choice by score + correction, weights from the scores alone,
-    renormalised and scaled (``ops.moe_route_biased``); then the chosen experts' two products over the (token,
+    renormalised and scaled (``ops.moe_route_biased``, or inside the one launch that a step of few tokens
+    needs for routing, sort and identity rows); then the chosen experts' two products over the (token,
     choice) pairs grouped by expert on the device, a pair that chose an identity expert contributing its token's
     row itself (``ops.moe_experts``).  The output is float32 [top, T, H] or [1, T, H], as GroupedMoE's."""
     graph_safe = True
@@ -135,12 +136,13 @@ class BiasedMoE:
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         s = self.spec
         logits = ops.gemm(x, self.w_router, out_dtype=torch.float32)
-        ids, weights = ops.moe_route_biased(logits, self.correction, s.top, s.route_scale)
+
         # (rows_in_activation_type: the experts' output rows of a long portion in bfloat16 instead of 32-bit before
         # they are weighed and added in 32-bit: 7 % less time for the down product and 18 % for the sum at 8192
         # pairs of width 2048, for one more rounding of every expert's output; off)
         rows = ctx.rt.dtype if self.rows_in_activation_type else torch.float32
-        return ops.moe_experts(x, ids, weights, self.w_up, self.w_down, act="relu_sq", identity=self.ident, rows_dtype=rows)
+        return ops.moe_experts(x, None, None, self.w_up, self.w_down, act="relu_sq", identity=self.ident, rows_dtype=rows,
+                               biased_route=(logits, self.correction, s.top, s.route_scale))
 
 
 register_part("polynorm_mlp", PolyNormMLP)

@@ -257,3 +257,22 @@ def test_squared_relu_experts_and_identity_experts_over_rows_grouped_on_the_devi
                                   rows_dtype=rows_dtype)
         assert parts.dtype == torch.float32 and parts.shape[1:] == (T, H)
         assert rel(parts.sum(0), want) < tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,H,Fd,E,ident,top", [(1, 128, 64, 8, 3, 2), (8, 256, 32, 32, 4, 4), (37, 96, 40, 6, 2, 3), (64, 64, 16, 70, 3, 5),
+                                                (5, 128, 64, 1, 1, 2), (3, 64, 8, 4, 0, 1)])
+def test_few_tokens_route_sort_and_identity_rows_in_one_launch(dtype, T, H, Fd, E, ident, top):
+    """A step of few tokens routes, sorts and writes the identity experts' rows in one launch: the same parts, bit for
+    bit, as the router's kernel, the sort's and the identity rows' one after the other."""
+    o = ops()
+    g = torch.Generator().manual_seed(T * 7 + E)
+    x = torch.randn(T, H, generator=g).to(dtype).to(DEV)
+    up = (torch.randn(E, Fd, H, generator=g) / math.sqrt(H)).to(dtype).to(DEV)
+    down = (torch.randn(E, H, Fd, generator=g) / math.sqrt(Fd)).to(dtype).to(DEV)
+    z = (torch.randn(T, E + ident, generator=g) * 2.0).to(DEV)
+    corr = (torch.randn(E + ident, generator=g) * 0.2).to(DEV)
+    ids, w = o.moe_route_biased(z, corr, top, 1.7)
+    want = o.moe_experts(x, ids, w, up, down, act="relu_sq", identity=ident)
+    got = o.moe_experts(x, None, None, up, down, act="relu_sq", identity=ident, biased_route=(z, corr, top, 1.7))
+    assert torch.equal(got, want)
