@@ -500,6 +500,14 @@ def gemm_branch_splits(x: torch.Tensor, w: torch.Tensor) -> int:
     return int(lib.qe_gemm_branch_splits(x.shape[0], w.shape[0], x.shape[1], _DT[x.dtype], _DT[w.dtype]))
 
 
+def gemm_branch_splits_for(rows: int, w: torch.Tensor, x_dtype: torch.dtype) -> int:
+    """gemm_branch_splits for ``rows`` rows of x_dtype that are yet to be computed."""
+    lib = load_library()
+    if x_dtype not in _DT or w.dtype not in _DT:
+        return 0
+    return int(lib.qe_gemm_branch_splits(int(rows), w.shape[0], w.shape[1], _DT[x_dtype], _DT[w.dtype]))
+
+
 def gemm_partial_preferred(x: torch.Tensor, w: torch.Tensor) -> bool:
     """True if the product of these operands is quickest cut along K into partial products
     (EPI_PARTIAL): more than 16 and at most 64 rows against a matrix of 16 M elements or more."""
@@ -1105,7 +1113,8 @@ def qkv_conv_rope_store(qkv: torch.Tensor, conv_w: torch.Tensor, state: Optional
 def moe_experts(x: torch.Tensor, ids: Optional[torch.Tensor], weights: Optional[torch.Tensor], w_gate_up: torch.Tensor,
                 w_down: torch.Tensor, limit: float = 0.0, slope: float = 1.0, interleaved: bool = False,
                 algo: int = ALGO_AUTO, act: str = "gated", identity: int = 0,
-                rows_dtype: torch.dtype = torch.float32, biased_route=None) -> torch.Tensor:
+                rows_dtype: torch.dtype = torch.float32, biased_route=None,
+                parts_out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The chosen experts' outputs, weighted: float32 [S, T, H] whose sum over S, in order, is the mixture's
     output (S = top: a token's choices in their order; or S = 1: already added up in that order).
     x [T, K]; w_gate_up [E, 2 F, K] (gate rows, then up rows; or, ``interleaved``, in alternating blocks of
@@ -1117,7 +1126,8 @@ def moe_experts(x: torch.Tensor, ids: Optional[torch.Tensor], weights: Optional[
     weighed and added in 32-bit (float32, or bfloat16 with bfloat16 operands: half the bytes of the largest tensor of
     the mixture).  ``biased_route``: instead of ids and weights (both None), (logits float32 [T, E + identity],
     correction float32 [E + identity], top, scale) for the routing of moe_route_biased: a step of few tokens then
-    routes, sorts and writes the identity experts' rows in one launch.
+    routes, sorts and writes the identity experts' rows in one launch.  ``parts_out``: float32 [top, T, H] to take the
+    parts (the paths of fewer than 1024 pairs only).
 
     The (token, choice) pairs are grouped by expert on the device.  bfloat16 with many pairs: their rows are
     gathered side by side and both products run on the tiled kernel of the dense products, a tile of 128
@@ -1168,6 +1178,11 @@ def moe_experts(x: torch.Tensor, ids: Optional[torch.Tensor], weights: Optional[
     perm, inv, tiles, n_tiles = meta[:n], meta[n:2 * n], meta[2 * n:2 * n + 3 * max_tiles], meta[2 * n + 3 * max_tiles:]
     fused_front = False
     parts = None
+    if parts_out is not None:
+        if tiled:
+            raise KernelError("moe_experts: parts_out goes with fewer than 1024 pairs")
+        _need(parts_out, "parts_out", torch.float32, (top, T, Hout), dev)
+        parts = parts_out
     if biased_route is not None:
         if r_logits.shape[1] != E + identity:
             raise KernelError(f"moe_experts: {r_logits.shape[1]} router outputs for {E} experts and {identity} identity experts")
@@ -1175,7 +1190,8 @@ def moe_experts(x: torch.Tensor, ids: Optional[torch.Tensor], weights: Optional[
             # few tokens: routing, sort and the identity experts' rows in one launch
             ids = torch.empty((T, top), dtype=torch.int32, device=dev)
             weights = torch.empty((T, top), dtype=torch.float32, device=dev)
-            parts = torch.empty((top, T, Hout), dtype=torch.float32, device=dev)
+            if parts is None:
+                parts = torch.empty((top, T, Hout), dtype=torch.float32, device=dev)
             _check(lib.qe_moe_front_small(r_logits.data_ptr(), r_corr.data_ptr(), x.data_ptr(), ids.data_ptr(),
                                           weights.data_ptr(), perm.data_ptr(), inv.data_ptr(), tiles.data_ptr(),
                                           n_tiles.data_ptr(), parts.data_ptr(), max_tiles, T, Hout, E + identity, E, top,

@@ -369,9 +369,14 @@ class ConvAttention(PagedAttention):
         if self.position is not None:
             self.position.load({}, rt)
 
-    def forward(self, x: torch.Tensor, ctx, binding: CacheBinding) -> torch.Tensor:
+    def output_parts(self, rows: int, dtype: torch.dtype) -> int:
+        """Into how many 32-bit partial products the output projection of ``rows`` rows is cut (0: not at all):
+        forward can leave them in a tensor it is given (``parts_out``)."""
+        return ops.gemm_branch_splits_for(rows, self.w_o, dtype)
+
+    def forward(self, x: torch.Tensor, ctx, binding: CacheBinding, parts_out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """x [T, H] in the activation type.  Returns the mixer's output [T, H], or float32 partial products
-        [S, T, H] of it."""
+        [S, T, H] of it (in ``parts_out`` [S, T, H], S = output_parts(T, type), if given)."""
         if binding.kv is None:
             raise RuntimeError("attention was given no cache")
         if self.taps > 1 and binding.state is None:
@@ -391,7 +396,10 @@ class ConvAttention(PagedAttention):
                           other_tiles=self._other_tiles(ctx) if ex["other_tokens"] is not None else None,
                           max_other_keys=ex.get("max_other_keys", 0), other_keys_row=ex.get("other_keys_row"),
                           shared_keys=ctx.shared_keys, keep_first=self.keep_first, sink=self.sink)
-        return self._project_out(o.view(T, self.hq * self.d))
+        o = o.view(T, self.hq * self.d)
+        if parts_out is not None:
+            return ops.gemm(o, self.w_o, epilogue=ops.EPI_PARTIAL, splits=parts_out.shape[0], out=parts_out)
+        return self._project_out(o)
 
 
 register_part("paged_attention", PagedAttention)

@@ -241,6 +241,16 @@ class ParallelBlock:
     def forward(self, h, pending: Optional[torch.Tensor], ctx, bindings):
         stream = h if isinstance(h, Stream) else Stream(h)
         n = self.norm.forward(stream.h, ctx.rt, delta=pending)
+        T = n.shape[0]
+        if self.ffn is not None and stream.spare is not None and hasattr(self.mixer, "output_parts") and \
+                hasattr(self.ffn, "output_parts"):
+            # few rows: both branches leave 32-bit parts, side by side in one tensor, which the next norm adds in order
+            sa, sf = self.mixer.output_parts(T, ctx.rt.dtype), self.ffn.output_parts(T)
+            if sa > 0 and sf > 0:
+                parts = torch.empty((sa + sf, T, self.hidden), dtype=torch.float32, device=n.device)
+                self.mixer.forward(n, ctx, bindings[0], parts_out=parts[:sa])
+                self.ffn.forward(n, ctx, parts_out=parts[sa:])
+                return parts
         a = self.mixer.forward(n, ctx, bindings[0])
         if self.ffn is None:
             return a

@@ -84,7 +84,12 @@ class GroupedMoE:
         per = (self.w_gate_up[0].numel() + self.w_down[0].numel()) * self.w_down.element_size()
         return min(self.e, tokens * self.top) * per + self.w_router.numel() * self.w_router.element_size()
 
-    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+    def output_parts(self, rows: int) -> int:
+        """How many 32-bit parts forward leaves for ``rows`` rows where it can write them into a tensor it is given
+        (``parts_out``); 0 where it cannot (many pairs: the sum is formed here)."""
+        return self.top if rows * self.top < 1024 else 0
+
+    def forward(self, x: torch.Tensor, ctx, parts_out: Optional[torch.Tensor] = None) -> torch.Tensor:
         s = self.spec
         logits = ops.gemm(x, self.w_router, out_dtype=torch.float32)
         ids, weights = ops.moe_route(logits, s.num_groups, s.keep_groups, s.top)
@@ -133,7 +138,12 @@ class BiasedMoE:
         per = (self.w_up[0].numel() + self.w_down[0].numel()) * self.w_down.element_size()
         return min(self.e, tokens * self.top) * per + self.w_router.numel() * self.w_router.element_size()
 
-    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+    def output_parts(self, rows: int) -> int:
+        """How many 32-bit parts forward leaves for ``rows`` rows where it can write them into a tensor it is given
+        (``parts_out``); 0 where it cannot (many pairs: the sum is formed here)."""
+        return self.top if rows * self.top < 1024 else 0
+
+    def forward(self, x: torch.Tensor, ctx, parts_out: Optional[torch.Tensor] = None) -> torch.Tensor:
         s = self.spec
         logits = ops.gemm(x, self.w_router, out_dtype=torch.float32)
 
@@ -142,7 +152,7 @@ class BiasedMoE:
         # pairs of width 2048, for one more rounding of every expert's output; off)
         rows = ctx.rt.dtype if self.rows_in_activation_type else torch.float32
         return ops.moe_experts(x, None, None, self.w_up, self.w_down, act="relu_sq", identity=self.ident, rows_dtype=rows,
-                               biased_route=(logits, self.correction, s.top, s.route_scale))
+                               biased_route=(logits, self.correction, s.top, s.route_scale), parts_out=parts_out)
 
 
 register_part("polynorm_mlp", PolyNormMLP)
