@@ -112,16 +112,16 @@ extern "C" int qe_moe_route(const float* logits, int* ids, float* weights, int T
 // (the barriers are the block's); a wave without a token (z null) only keeps step.
 __device__ __forceinline__ void route_biased_token(const float* __restrict__ z, const float* __restrict__ correction,
                                                    float* sc, int* __restrict__ ids, float* __restrict__ weights, int E,
-                                                   int top, float scale, int lane) {
+                                                   int top, float scale, int lane, long zs = 1) {
     float* ch = sc + E;
     float* picked = ch + E;
-    if (z) {
+    if (z) {                                             // (zs: the distance between a token's logits)
         float mx = -INFINITY;
-        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e * zs]);
         mx = wave_max(mx);
         float sum = 0.f;
         for (int e = lane; e < E; e += 64) {
-            const float ex = expf(z[e] - mx);
+            const float ex = expf(z[e * zs] - mx);
             sc[e] = ex;
             sum += ex;
         }
@@ -160,18 +160,20 @@ __device__ __forceinline__ void route_biased_token(const float* __restrict__ z, 
 
 __global__ __launch_bounds__(64) void moe_route_biased_kernel(const float* __restrict__ logits, const float* __restrict__ correction,
                                                               int* __restrict__ ids, float* __restrict__ weights, int E, int top,
-                                                              float scale) {
+                                                              float scale, int transposed) {
     extern __shared__ float sc[];          // E scores, E choice scores, top chosen scores
     const long t = blockIdx.x;
-    route_biased_token(logits + t * E, correction, sc, ids + t * top, weights + t * top, E, top, scale, threadIdx.x);
+    // (transposed: logits [E, T], as a product of the router's few rows against the tokens' many leaves them)
+    route_biased_token(transposed ? logits + t : logits + t * E, correction, sc, ids + t * top, weights + t * top, E, top,
+                       scale, threadIdx.x, transposed ? (long)gridDim.x : 1L);
 }
 
 extern "C" int qe_moe_route_biased(const float* logits, const float* correction, int* ids, float* weights, int T, int E,
-                                   int top, float scale, hipStream_t stream) {
+                                   int top, float scale, int transposed, hipStream_t stream) {
     QE_REQUIRE(T >= 0 && E > 0 && top >= 1 && top <= E, "moe_route_biased: top %d of %d experts", top, E);
     QE_REQUIRE((2 * E + top) * sizeof(float) <= 60000, "moe_route_biased: too many experts");
     if (T == 0) return 0;
-    moe_route_biased_kernel<<<T, 64, (2 * E + top) * sizeof(float), stream>>>(logits, correction, ids, weights, E, top, scale);
+    moe_route_biased_kernel<<<T, 64, (2 * E + top) * sizeof(float), stream>>>(logits, correction, ids, weights, E, top, scale, transposed);
     QE_LAUNCH_CHECK();
     return 0;
 }

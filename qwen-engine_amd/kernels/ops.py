@@ -78,7 +78,7 @@ def load_library():
         "qe_attention": [vp, vp, vp, vp, vp, vp, i32, vp, i32, i32, i32, i32, i32, f32, i32, i32, i32, i32, vp],
         "qe_qkv_conv_rope_store": [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, vp],
         "qe_scale_f32": [vp, i64, f32, vp],
-        "qe_moe_route_biased": [vp, vp, vp, vp, i32, i32, i32, f32, vp],
+        "qe_moe_route_biased": [vp, vp, vp, vp, i32, i32, i32, f32, i32, vp],
         "qe_moe_front_small_supported": [i32, i32, i32],
         "qe_moe_front_small": [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, i32, vp],
         "qe_moe_identity": [vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp],
@@ -1043,18 +1043,18 @@ def moe_route(logits: torch.Tensor, groups: int, keep: int, top: int):
     return ids, weights
 
 
-def moe_route_biased(logits: torch.Tensor, correction: torch.Tensor, top: int, scale: float):
-    """logits float32 [T, E], correction float32 [E] -> (ids int32 [T, top], weights float32 [T, top]): softmax
+def moe_route_biased(logits: torch.Tensor, correction: torch.Tensor, top: int, scale: float, transposed: bool = False):
+    """logits float32 [T, E] (``transposed``: [E, T]), correction float32 [E] -> (ids int32 [T, top], weights float32 [T, top]): softmax
     over all experts; the ``top`` largest of score + correction are chosen (the lower index on ties); their
     weights are their scores without the correction, divided by the chosen scores' sum (+ 1e-20), times scale."""
     lib = load_library()
     _need(logits, "logits", torch.float32, (None, None))
-    T, E = logits.shape
+    T, E = (logits.shape[1], logits.shape[0]) if transposed else logits.shape
     _need(correction, "correction", torch.float32, (E,), logits.device)
     ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
     _check(lib.qe_moe_route_biased(logits.data_ptr(), correction.data_ptr(), ids.data_ptr(), weights.data_ptr(), T, E,
-                                   int(top), float(scale), _stream()), "moe_route_biased")
+                                   int(top), float(scale), int(bool(transposed)), _stream()), "moe_route_biased")
     return ids, weights
 
 
@@ -1125,7 +1125,8 @@ def moe_experts(x: torch.Tensor, ids: Optional[torch.Tensor], weights: Optional[
     ``rows_dtype``: the element type in which the path of many pairs leaves an expert's output rows before they are
     weighed and added in 32-bit (float32, or bfloat16 with bfloat16 operands: half the bytes of the largest tensor of
     the mixture).  ``biased_route``: instead of ids and weights (both None), (logits float32 [T, E + identity],
-    correction float32 [E + identity], top, scale) for the routing of moe_route_biased: a step of few tokens then
+    correction float32 [E + identity], top, scale[, transposed: the logits are [E + identity, T]]) for the routing of
+    moe_route_biased: a step of few tokens then
     routes, sorts and writes the identity experts' rows in one launch.  ``parts_out``: float32 [top, T, H] to take the
     parts (the paths of fewer than 1024 pairs only).
 
@@ -1141,10 +1142,12 @@ def moe_experts(x: torch.Tensor, ids: Optional[torch.Tensor], weights: Optional[
     if biased_route is not None:
         if ids is not None or weights is not None:
             raise KernelError("moe_experts: ids and weights, or a route to compute them, not both")
-        r_logits, r_corr, top, r_scale = biased_route
+        r_logits, r_corr, top, r_scale = biased_route[:4]
+        r_transposed = len(biased_route) > 4 and bool(biased_route[4])       # logits [E + identity, T]
         top = int(top)
-        _need(r_logits, "logits", torch.float32, (T, None), dev)
-        _need(r_corr, "correction", torch.float32, (r_logits.shape[1],), dev)
+        _need(r_logits, "logits", torch.float32, (None, T) if r_transposed else (T, None), dev)
+        r_outputs = r_logits.shape[0] if r_transposed else r_logits.shape[1]
+        _need(r_corr, "correction", torch.float32, (r_outputs,), dev)
     else:
         _need(ids, "ids", torch.int32, (T, None), dev)
         top = ids.shape[1]
@@ -1184,9 +1187,9 @@ def moe_experts(x: torch.Tensor, ids: Optional[torch.Tensor], weights: Optional[
         _need(parts_out, "parts_out", torch.float32, (top, T, Hout), dev)
         parts = parts_out
     if biased_route is not None:
-        if r_logits.shape[1] != E + identity:
-            raise KernelError(f"moe_experts: {r_logits.shape[1]} router outputs for {E} experts and {identity} identity experts")
-        if not tiled and lib.qe_moe_front_small_supported(T, E + identity, top):
+        if r_outputs != E + identity:
+            raise KernelError(f"moe_experts: {r_outputs} router outputs for {E} experts and {identity} identity experts")
+        if not tiled and not r_transposed and lib.qe_moe_front_small_supported(T, E + identity, top):
             # few tokens: routing, sort and the identity experts' rows in one launch
             ids = torch.empty((T, top), dtype=torch.int32, device=dev)
             weights = torch.empty((T, top), dtype=torch.float32, device=dev)
@@ -1198,7 +1201,7 @@ def moe_experts(x: torch.Tensor, ids: Optional[torch.Tensor], weights: Optional[
                                           float(r_scale), tile_rows, _DT[x.dtype], _stream()), "moe_front_small")
             fused_front = True
         else:
-            ids, weights = moe_route_biased(r_logits, r_corr, top, r_scale)
+            ids, weights = moe_route_biased(r_logits, r_corr, top, r_scale, transposed=r_transposed)
     # (identity experts are buckets of the sort like the others, behind them, and get no tiles)
     if not fused_front:
         _check(lib.qe_moe_sort(ids.data_ptr(), n, E + identity, E, tile_rows, perm.data_ptr(), inv.data_ptr(), tiles.data_ptr(),

@@ -374,9 +374,12 @@ class ConvAttention(PagedAttention):
         forward can leave them in a tensor it is given (``parts_out``)."""
         return ops.gemm_branch_splits_for(rows, self.w_o, dtype)
 
-    def forward(self, x: torch.Tensor, ctx, binding: CacheBinding, parts_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, ctx, binding: CacheBinding, parts_out: Optional[torch.Tensor] = None,
+                add_to: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """x [T, H] in the activation type.  Returns the mixer's output [T, H], or float32 partial products
-        [S, T, H] of it (in ``parts_out`` [S, T, H], S = output_parts(T, type), if given)."""
+        [S, T, H] of it (in ``parts_out`` [S, T, H], S = output_parts(T, type), if given).  ``add_to``: the 32-bit
+        stream [T, H]; where the output projection can add its result into it itself (its residual epilogue, and
+        no cut along K wanted) it does, and None is returned: nothing is left to add."""
         if binding.kv is None:
             raise RuntimeError("attention was given no cache")
         if self.taps > 1 and binding.state is None:
@@ -399,6 +402,9 @@ class ConvAttention(PagedAttention):
         o = o.view(T, self.hq * self.d)
         if parts_out is not None:
             return ops.gemm(o, self.w_o, epilogue=ops.EPI_PARTIAL, splits=parts_out.shape[0], out=parts_out)
+        if add_to is not None and not ops.gemm_branch_splits(o, self.w_o) and ops.gemm_fused_supported(o, self.w_o):
+            ops.gemm(o, self.w_o, epilogue=ops.EPI_RESIDUAL, out=add_to)
+            return None
         return self._project_out(o)
 
 

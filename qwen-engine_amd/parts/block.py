@@ -251,10 +251,16 @@ class ParallelBlock:
                 self.mixer.forward(n, ctx, bindings[0], parts_out=parts[:sa])
                 self.ffn.forward(n, ctx, parts_out=parts[sa:])
                 return parts
-        a = self.mixer.forward(n, ctx, bindings[0])
+        if self.ffn is not None and hasattr(self.mixer, "output_parts"):
+            # (the mixer's last product adds into the stream itself where it can: the feed-forward reads n, not the stream)
+            a = self.mixer.forward(n, ctx, bindings[0], add_to=stream.h)
+        else:
+            a = self.mixer.forward(n, ctx, bindings[0])
         if self.ffn is None:
             return a
         y = self.ffn.forward(n, ctx)
+        if a is None:
+            return y
         if a.dim() == 3 and y.dim() == 3 and a.dtype == y.dtype:
             # both branches left 32-bit parts (few rows): one list of parts, added in order by the next norm
             return torch.cat([a, y], dim=0)

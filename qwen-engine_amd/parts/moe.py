@@ -145,14 +145,18 @@ class BiasedMoE:
 
     def forward(self, x: torch.Tensor, ctx, parts_out: Optional[torch.Tensor] = None) -> torch.Tensor:
         s = self.spec
-        logits = ops.gemm(x, self.w_router, out_dtype=torch.float32)
-
+        # Many rows against the router's few: the product the other way round, logits^T = W_router x^T, is a product of
+        # few rows against a large matrix, which fills the chip where the router's few outputs give a handful of tiles;
+        # the logits are 32-bit sums of the same products either way.
+        transposed = x.shape[0] > 64 and self.w_router.shape[0] <= 64
+        logits = ops.gemm(self.w_router, x, out_dtype=torch.float32) if transposed else \
+            ops.gemm(x, self.w_router, out_dtype=torch.float32)
         # (rows_in_activation_type: the experts' output rows of a long portion in bfloat16 instead of 32-bit before
         # they are weighed and added in 32-bit: 7 % less time for the down product and 18 % for the sum at 8192
         # pairs of width 2048, for one more rounding of every expert's output; off)
         rows = ctx.rt.dtype if self.rows_in_activation_type else torch.float32
         return ops.moe_experts(x, None, None, self.w_up, self.w_down, act="relu_sq", identity=self.ident, rows_dtype=rows,
-                               biased_route=(logits, self.correction, s.top, s.route_scale), parts_out=parts_out)
+                               biased_route=(logits, self.correction, s.top, s.route_scale, transposed), parts_out=parts_out)
 
 
 register_part("polynorm_mlp", PolyNormMLP)

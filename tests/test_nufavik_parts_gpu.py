@@ -227,6 +227,8 @@ def test_router_chooses_by_corrected_scores_and_weighs_by_the_scores(E, top, sca
         wi, ww = N.route(z[t].double(), corr.double(), top, scale)
         assert ids[t].tolist() == wi, t
         assert rel(w[t], ww) < 1e-5
+    ids_t, w_t = ops().moe_route_biased(z.t().contiguous().to(DEV), corr.to(DEV), top, scale, transposed=True)
+    assert torch.equal(ids_t, ids) and torch.equal(w_t, w)            # (the logits the other way round: the same bits)
     ids, w = ops().moe_route_biased(torch.zeros(2, E, device=DEV), torch.zeros(E, device=DEV), top, scale)
     assert ids[1].tolist() == list(range(top))            # ties: the lower index
     assert rel(w[1], torch.full((top,), scale / top, dtype=torch.float64)) < 1e-5
