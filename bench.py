@@ -378,10 +378,10 @@ def nufavik_config(z, layers, vocab):
     layer = {"type": "attention",
              "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"], "conv": z["conv"],
                        "scale": z["dim"] ** -0.5, "mask": {"size": z["window"], "keep_first": z["keep_first"]},
-                       "rot": {"base": 1000000.0, "dims": z["rot_dims"]}},
+                       "rot": {"base": 10000.0, "dims": z["rot_dims"]}},
              "mlp": {"kind": "moe", "expert": {"ff": z["expert_ff"]},
-                     "router": {"experts": z["experts"], "identity": z["identity"], "top": z["top"], "scale": 1.5}}}
-    return {"architecture": "Nufavik", "vocab": vocab, "width": z["width"], "embedding": {"scale": 0.5}, "norm": {"eps": 1e-5},
+                     "router": {"experts": z["experts"], "identity": z["identity"], "top": z["top"], "scale": 2.0}}}
+    return {"architecture": "Nufavik", "vocab": vocab, "width": z["width"], "embedding": {"scale": 0.8}, "norm": {"eps": 1e-6},
             "layers": [layer] * layers}
 
 

@@ -261,9 +261,6 @@ class ParallelBlock:
         y = self.ffn.forward(n, ctx)
         if a is None:
             return y
-        if a.dim() == 3 and y.dim() == 3 and a.dtype == y.dtype:
-            # both branches left 32-bit parts (few rows): one list of parts, added in order by the next norm
-            return torch.cat([a, y], dim=0)
         ops.residual_add(stream.h, a)
         return y
 

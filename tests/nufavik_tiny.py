@@ -24,7 +24,7 @@ def _moe(experts, identity, top, ff, scale):
 # within a page, beyond one, and more than the window is long
 NA = {"architecture": "Nufavik", "vocab": 211, "width": 96, "embedding": {"scale": 0.7}, "norm": {"eps": 1e-6},
       "layers": [
-          _layer(4, 2, 16, 24, 3, 24, 3, 8, 0.3, 1000.0, _moe(6, 2, 2, 40, 1.5)),
+          _layer(4, 2, 16, 24, 3, 24, 3, 8, 0.3, 1000.0, _moe(6, 2, 2, 40, 1.25)),
           _layer(3, 3, 24, 8, 2, 7, 0, 24, 0.25, 50000.0, None),
           _layer(6, 1, 8, 40, 5, 37, 20, 0, 0.4, 100.0, _moe(3, 1, 3, 24, 0.8)),
           _layer(2, 1, 32, 16, 4, 9, 12, 2, 0.2, 10.0, _moe(5, 0, 1, 56, 2.0)),
@@ -32,7 +32,7 @@ NA = {"architecture": "Nufavik", "vocab": 211, "width": 96, "embedding": {"scale
 # B: sizes that fill whole tiles of the matrix-unit kernels (heads of 64 and 128, groups of 4 and 1)
 NB = {"architecture": "Nufavik", "vocab": 300, "width": 128, "embedding": {"scale": 2.0}, "norm": {"eps": 1e-5},
       "layers": [
-          _layer(8, 2, 64, 64, 4, 33, 5, 32, 0.11, 1000000.0, _moe(8, 0, 1, 64, 1.0)),
+          _layer(8, 2, 64, 64, 4, 33, 5, 16, 0.11, 500000.0, _moe(8, 0, 1, 64, 1.0)),
           _layer(4, 4, 128, 96, 3, 100, 17, 64, 0.08, 10000.0, _moe(4, 3, 3, 128, 2.5)),
       ]}
 # C: values that are 1 or equal: embedding scale 1, route scale 1, one head, keys and values of one size, one expert

@@ -256,7 +256,7 @@ def test_command_line_with_random_weights(tmp_path, capsys):
 NM = {"architecture": "Nufavik", "vocab": 701, "width": 320, "embedding": {"scale": 1.3}, "norm": {"eps": 1e-5},
       "layers": [
           {"type": "attention",
-           "mixer": {"heads": 6, "kv_heads": 2, "dim": 64, "vdim": 48, "conv": 3, "scale": 0.12,
+           "mixer": {"heads": 6, "kv_heads": 2, "dim": 64, "vdim": 40, "conv": 5, "scale": 0.12,
                      "mask": {"size": 150, "keep_first": 40}, "rot": {"base": 20000.0, "dims": 24}},
            "mlp": {"kind": "moe", "expert": {"ff": 64}, "router": {"experts": 12, "identity": 2, "top": 3, "scale": 1.7}}},
           {"type": "attention",

@@ -139,7 +139,7 @@ def _plain_attention(q, k, v, pos, scale, size, keep, sink):
 
 
 CASES = [  # window, kept first keys, sink
-    (40, 4, True), (40, 0, True), (0, 0, True), (16, 16, False), (17, 33, True), (150, 140, True), (1, 1, True),
+    (41, 5, True), (41, 0, True), (0, 0, True), (16, 16, False), (17, 33, True), (150, 140, True), (1, 1, True),
     (300, 7, False), (64, 130, True), (5, 40, True),
 ]
 
